@@ -157,6 +157,36 @@ LISORAX_PRESETS: dict[str, dict] = {
 }
 
 
+def _mozidra(width: int, heads: int, kv_heads: int, n_layers: int, vocab: int, ff: int, experts: int = 8,
+             top: int = 2, streams: int = 4, attn_every: int = 3, window: int = 1024) -> dict:
+    """A Mozidra config dict at transformer-like sizes: 128-dim heads; every ``attn_every``-th layer grouped-query
+    attention with a full rotation and value mixing, the others latent attention (rank 512); sliding windows; every
+    layer with group-routed experts of ``ff`` rows (4 groups, 2 kept) and a shared expert of the same size."""
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4 if experts % 4 == 0 else 1,
+                                                                 "keep": 2 if experts % 4 == 0 else 1}},
+           "shared": {"ff": ff, "limit": 7.0}}
+    layers = []
+    for i in range(n_layers):
+        if i % attn_every == attn_every - 1:
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                 "mask": {"size": 2 * window}, "rot": {"base": 500000.0, "dims": 128}, "v_mix": True}
+            layers.append({"type": "attention", "mixer": m, "mlp": moe})
+        else:
+            m = {"heads": heads, "dim": 128, "vdim": 128, "kv_rank": 512, "scale": 128 ** -0.5,
+                 "mask": {"size": window}}
+            layers.append({"type": "latent_attention", "mixer": m, "mlp": moe})
+    return {"architecture": "Mozidra", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "streams": streams}
+
+
+MOZIDRA_PRESETS: dict[str, dict] = {
+    # widths, heads and vocabularies of the Llama presets above; 8 experts of ff / 4 rows, top 2 (random init)
+    "mozidra-small": _mozidra(1024, 16, 4, 6, 128256, 896),
+    "mozidra-tiny": _mozidra(512, 8, 2, 3, 32000, 256, experts=4, window=64),
+}
+
+
 def _budurax_config(c: dict, name: str):
     from kafka_llm_service_amd.models.budurax import BuduraxConfig
 
@@ -169,15 +199,21 @@ def _lisorax_config(c: dict, name: str):
     return LisoraxConfig.from_dict(c, name=name)
 
 
+def _mozidra_config(c: dict, name: str):
+    from kafka_llm_service_amd.models.mozidra import MozidraConfig
+
+    return MozidraConfig.from_dict(c, name=name)
+
+
 # config.json "architecture" (lower case) -> config class of a model family that names itself there
-ARCH_CONFIGS = {"budurax": _budurax_config, "lisorax": _lisorax_config}
+ARCH_CONFIGS = {"budurax": _budurax_config, "lisorax": _lisorax_config, "mozidra": _mozidra_config}
 # model families whose kernels are built for float32 as well as bfloat16 (EngineConfig.dtype)
-FP32_ARCHS = ("budurax", "lisorax")
+FP32_ARCHS = ("budurax", "lisorax", "mozidra")
 
 
 def _from_json(path: Path):
     """A config.json names its model class: ``"architecture": "Budurax"`` (models/budurax.py), ``"Lisorax"``
-    (models/lisorax.py), else HF Llama / Mixtral."""
+    (models/lisorax.py), ``"Mozidra"`` (models/mozidra.py), else HF Llama / Mixtral."""
     c = json.loads(path.read_text())
     make = ARCH_CONFIGS.get(str(c.get("architecture", "")).lower())
     if make is not None:
@@ -192,9 +228,11 @@ def get_config(name: str):
         return _budurax_config(BUDURAX_PRESETS[name], name)
     if name in LISORAX_PRESETS:
         return _lisorax_config(LISORAX_PRESETS[name], name)
+    if name in MOZIDRA_PRESETS:
+        return _mozidra_config(MOZIDRA_PRESETS[name], name)
     p = Path(name)
     if p.is_dir() and (p / "config.json").exists():
         return _from_json(p / "config.json")
     if p.suffix == ".json" and p.exists():
         return _from_json(p)
-    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS) + sorted(BUDURAX_PRESETS) + sorted(LISORAX_PRESETS)}")
+    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS) + sorted(BUDURAX_PRESETS) + sorted(LISORAX_PRESETS) + sorted(MOZIDRA_PRESETS)}")

@@ -415,8 +415,10 @@ __device__ __forceinline__ float wave_allsum(float v) {
 
 // One wave per (row t, group of RPW heads). Lane l holds dimensions l, l + 64, ... of the query rows, of the key row
 // being visited and of the output accumulators; a key row is loaded once for the wave's heads, and its latent part
-// is also the value row. Keys are visited in order 0 .. position, KB at a time, whatever the step's batch: a row's
-// result does not depend on what else runs.
+// is also the value row. Keys are visited in order first visible .. position, KB at a time, whatever the step's batch:
+// a row's result does not depend on what else runs. window > 0: the row sees the last `window` keys up to its own
+// position only. sink != nullptr: head h's softmax denominator also holds e^(sink[h]) (the running maximum and sum
+// start from that term instead of from nothing).
 template <typename AT, int MAXC, int RPW, int KB>
 __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__ q_lat, int64_t ql_h, int64_t ql_t,
                                                           const AT* __restrict__ q_rot, int64_t qr_t, int64_t qr_h,
@@ -425,7 +427,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__
                                                           const int* __restrict__ tok_seg,
                                                           const int64_t* __restrict__ positions, float scale_log2e,
                                                           AT* __restrict__ out, int64_t o_h, int64_t o_t, int T, int H,
-                                                          int n_hg) {
+                                                          int n_hg, int window, const float* __restrict__ sink) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t task = (int64_t)blockIdx.x * 4 + wave;
   if (task >= (int64_t)T * n_hg) return;
@@ -438,6 +440,10 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__
   for (int r = 0; r < RPW; ++r) {
     m[r] = -INFINITY;
     l[r] = 0.f;
+    if (sink != nullptr && r < nh) {
+      m[r] = sink[h0 + r] * 1.4426950408889634f;
+      l[r] = 1.f;
+    }
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
       const int dim = lane + 64 * c;
@@ -451,7 +457,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const AT* __restrict__
   }
   const int nkeys = (int)positions[t] + 1;
   const int* btr = bt + (int64_t)tok_seg[t] * bt_stride;
-  for (int j0 = 0; j0 < nkeys; j0 += KB) {
+  const int jlo = window > 0 ? max(0, nkeys - window) : 0;
+  for (int j0 = jlo; j0 < nkeys; j0 += KB) {
     float k[KB][MAXC];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
@@ -529,7 +536,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     int64_t qr_h, const bf16* __restrict__ cache, const bf16* __restrict__ cache_t, int R, int rd,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
     float scale_log2e, bf16* __restrict__ out, int64_t o_h, int64_t o_t, int H, float* __restrict__ po,
-    float* __restrict__ pml, int T) {
+    float* __restrict__ pml, int T, int window, const float* __restrict__ sink) {
+  // window > 0: a row at position p sees the keys p - window < j <= p; the tile starts at the key block that holds
+  // the first key its first row sees. sink != nullptr: head h's denominator also holds e^(sink[h]) (added once, at
+  // the end here or in latent_merge).
   // gridDim.z > 1: the tile's key blocks are dealt to gridDim.z workgroups in contiguous ranges; each leaves its
   // unnormalised accumulators in po [z][H][T][R] and (row maximum, row sum) in pml [z][H][T][2] for latent_merge
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -578,6 +588,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < 16; ++i) O[tw][i] = 0.f;
   const int* btr = bt + (int64_t)sg * bt_stride;
   const int nblocks = (maxpos >> 7) + 1;
+  const int kbmin = window > 0 ? max(0, (int)positions[t0] - window + 1) >> 7 : 0;
   const bf16* qrow = Qs + lr * qstride + 8 * lh;
   // this wave's key row of a block, all its 16-dim steps in flight at once (one memory round trip per block); the
   // next block's row is requested right after this block's score MFMAs, so it arrives under the softmax and the
@@ -592,8 +603,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       if (ks < nks) kf[ks] = load_bf16x8(krow + 16 * ks);
   };
   const int nsplit = gridDim.z;
-  const int bps = (nblocks + nsplit - 1) / nsplit;
-  const int kb0 = blockIdx.z * bps, kb1 = min(nblocks, kb0 + bps);
+  const int bps = (nblocks - kbmin + nsplit - 1) / nsplit;
+  const int kb0 = kbmin + blockIdx.z * bps, kb1 = min(nblocks, kb0 + bps);
   if (kb0 < kb1 && kb0 * 128 + 32 * w <= maxpos) fetch_keys(kb0);
   for (int kb = kb0; kb < kb1; ++kb) {
     // ---- scores of this wave's 32 keys
@@ -611,7 +622,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float s[16], mx[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      s[i] = (any && key <= prow[i]) ? S[i] * scale_log2e : -INFINITY;
+      s[i] = (any && key <= prow[i] && (window == 0 || key > prow[i] - window)) ? S[i] * scale_log2e : -INFINITY;
       float v = s[i];
 #pragma unroll
       for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
@@ -683,9 +694,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int i = 0; i < 16; ++i) {
     const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
     if (r >= nrows) continue;
-    const float l = mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r];
+    float l = mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r];
     const int64_t t = t0 + r / hpr, h = h0 + r % hpr;
     if (nsplit == 1) {
+      if (sink != nullptr) l += fast_exp2(sink[h] * 1.4426950408889634f - m[i]);
       const float inv = 1.0f / l;
 #pragma unroll
       for (int tw = 0; tw < TW; ++tw) {
@@ -709,7 +721,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
 // out[h][t] = sum_z 2^(m_z - m) O_z / sum_z 2^(m_z - m) l_z over the key-range splits of latent_attn_mfma_kernel
 __global__ void latent_merge_kernel(const float* __restrict__ po, const float* __restrict__ pml, int nsplit, int H,
-                                    int T, int R, bf16* __restrict__ out, int64_t o_h, int64_t o_t) {
+                                    int T, int R, bf16* __restrict__ out, int64_t o_h, int64_t o_t,
+                                    const float* __restrict__ sink) {
   const int64_t ht = blockIdx.x;  // h * T + t
   const int h = (int)(ht / T), t = (int)(ht - (int64_t)h * T);
   float mx = -INFINITY;
@@ -719,6 +732,7 @@ __global__ void latent_merge_kernel(const float* __restrict__ po, const float* _
     const float mz = pml[2 * ((int64_t)z * H * T + ht)];
     if (mz != -INFINITY) den += fast_exp2(mz - mx) * pml[2 * ((int64_t)z * H * T + ht) + 1];
   }
+  if (sink != nullptr) den += fast_exp2(sink[h] * 1.4426950408889634f - mx);
   const float inv = 1.0f / den;
   for (int d = threadIdx.x; d < R; d += blockDim.x) {
     float a = 0.f;
@@ -1186,8 +1200,9 @@ int kafka_hy_latent_attn_max_dk() { return 640; }
 hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
                                 int64_t qr_h, const void* cache, int page, int R, int rd, const int* bt, int bt_stride,
                                 const int* tok_seg, const int64_t* positions, float scale, void* out, int64_t o_h,
-                                int64_t o_t, int T, int H, hipStream_t st) {
+                                int64_t o_t, int T, int H, int window, const float* sink, hipStream_t st) {
   if (T <= 0) return hipSuccess;
+  if (window < 0) return hipErrorInvalidValue;
   constexpr int RPW = 4;
   const int n_hg = (H + RPW - 1) / RPW;
   const int64_t tasks = (int64_t)T * n_hg;
@@ -1197,7 +1212,7 @@ hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_
   DISPATCH_AT(f32, {
     auto a = [&](auto k) {
       k<<<grid, 256, 0, st>>>((const AT*)q_lat, ql_h, ql_t, (const AT*)q_rot, qr_t, qr_h, (const AT*)cache, page, R, rd,
-                              bt, bt_stride, tok_seg, positions, sl, (AT*)out, o_h, o_t, T, H, n_hg);
+                              bt, bt_stride, tok_seg, positions, sl, (AT*)out, o_h, o_t, T, H, n_hg, window, sink);
     };
     if (Dk <= 192) a(latent_attn_kernel<AT, 3, RPW, 4>);
     else if (Dk <= 384) a(latent_attn_kernel<AT, 6, RPW, 4>);
@@ -1216,8 +1231,10 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
                                      int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
                                      const int* bt, int bt_stride, const int* items, int n_items,
                                      const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
-                                     int nsplit, float* po, float* pml, int T, hipStream_t st) {
+                                     int nsplit, float* po, float* pml, int T, int window, const float* sink,
+                                     hipStream_t st) {
   if (n_items <= 0) return hipSuccess;
+  if (window < 0) return hipErrorInvalidValue;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (po == nullptr || pml == nullptr))) return hipErrorInvalidValue;
   if (!kafka_hy_latent_mfma_ok(16, R, rd)) return hipErrorInvalidValue;
   const int Dk = R + rd;
@@ -1228,7 +1245,7 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
   auto a = [&](auto k) {
     k<<<grid, 256, lds, st>>>((const bf16*)q_lat, ql_h, ql_t, (const bf16*)q_rot, qr_t, qr_h, (const bf16*)cache,
                               (const bf16*)cache_t, R, rd, bt, bt_stride, items, positions, sl, (bf16*)out, o_h, o_t, H,
-                              po, pml, T);
+                              po, pml, T, window, sink);
   };
   const int nks = Dk / 16;
   if (tw == 1 && nks <= 12) a(latent_attn_mfma_kernel<1, 12>);
@@ -1239,7 +1256,8 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
   else if (nks <= 36) a(latent_attn_mfma_kernel<4, 36>);
   else a(latent_attn_mfma_kernel<4, 40>);
   if (nsplit > 1)
-    latent_merge_kernel<<<(unsigned)((int64_t)H * T), 128, 0, st>>>(po, pml, nsplit, H, T, R, (bf16*)out, o_h, o_t);
+    latent_merge_kernel<<<(unsigned)((int64_t)H * T), 128, 0, st>>>(po, pml, nsplit, H, T, R, (bf16*)out, o_h, o_t,
+                                                                    sink);
   return hipGetLastError();
 }
 

@@ -26,14 +26,15 @@ hipError_t kafka_hy_latent_attn_mfma(const void* q_lat, int64_t ql_h, int64_t ql
                                      int64_t qr_h, const void* cache, const void* cache_t, int R, int rd,
                                      const int* bt, int bt_stride, const int* items, int n_items,
                                      const int64_t* positions, float scale, void* out, int64_t o_h, int64_t o_t, int H,
-                                     int nsplit, float* po, float* pml, int T, hipStream_t st);
+                                     int nsplit, float* po, float* pml, int T, int window, const float* sink,
+                                     hipStream_t st);
 hipError_t kafka_hy_sigmoid_mul(int f32, const void* a, int64_t a_h, int64_t a_t, const void* g, int64_t gs, void* out,
                                 int64_t T, int H, int vd, hipStream_t st);
 int kafka_hy_latent_attn_max_dk();
 hipError_t kafka_hy_latent_attn(int f32, const void* q_lat, int64_t ql_h, int64_t ql_t, const void* q_rot, int64_t qr_t,
                                 int64_t qr_h, const void* cache, int page, int R, int rd, const int* bt, int bt_stride,
                                 const int* tok_seg, const int64_t* positions, float scale, void* out, int64_t o_h,
-                                int64_t o_t, int T, int H, hipStream_t st);
+                                int64_t o_t, int T, int H, int window, const float* sink, hipStream_t st);
 hipError_t kafka_hy_short_conv(int f32, const void* proj, int64_t ps, int c0, const void* w, const void* b, int C,
                                int taps, const int* tok_seg, const int* seg, int R, void* state, void* out, int64_t T,
                                int silu, int residual, hipStream_t st);
@@ -87,9 +88,35 @@ hipError_t kafka_hy_moe_topk(const float* logits, int64_t ls, int E, int k, floa
 int kafka_hy_moe_rows_max_d();
 hipError_t kafka_hy_moe_rows(int f32, const void* h, int64_t hs, const void* wgu, const void* wd, const float* tw,
                              const int* te, int d, int F, int k, void* a, float* out, int64_t os, int64_t T,
-                             hipStream_t st);
+                             float limit, float alpha, hipStream_t st);
 hipError_t kafka_hy_add2(int f32, float* x, int64_t xs, const void* y1, int64_t s1, const void* y2, int64_t s2,
                          int y2_f32, int64_t T, int d, const void* w, float eps, void* out, int64_t os, hipStream_t st);
+
+// residual streams, windowed attention, group-limited router (hybrid_streams.hip)
+int kafka_hy_stream_max();
+hipError_t kafka_hy_stream_step(float* xs, int64_t s_stride, int64_t t_stride, int S, const void* y, int64_t ys,
+                                int y_f32, const void* y2, int64_t y2s, int y2_f32, const float* row_scale,
+                                const float* mix, const float* wr, const float* rd, const float* nw, float eps,
+                                void* out, int64_t os, int out_f32, float* total, int64_t ts, int64_t T, int d,
+                                hipStream_t st);
+hipError_t kafka_hy_swish_clamp_mul(int f32, const void* gu, int64_t gs, void* out, int64_t os, int64_t T, int F,
+                                    float limit, float alpha, hipStream_t st);
+hipError_t kafka_hy_qk_norm_rope_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
+                                       const float* qw, const float* kw, float eps, const int64_t* positions,
+                                       const float* cos_sin, int dims, const void* vf, int64_t vfs, int vf_off,
+                                       float lam, void* kc, void* vt, const int64_t* slots, void* q_out, int64_t qos,
+                                       int64_t T, hipStream_t st);
+int kafka_hy_window_attn_max_d();
+int kafka_hy_window_attn_max_dv();
+hipError_t kafka_hy_window_attn(int f32, const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
+                                int bt_stride, const int* tok_seg, const int64_t* positions, int H, int G, int D,
+                                int Dv, float scale, int window, const float* sink, void* out, int64_t os, int64_t T,
+                                hipStream_t st);
+int kafka_hy_grouped_router_max_e();
+int kafka_hy_grouped_router_max_k();
+int kafka_hy_grouped_router_max_g();
+hipError_t kafka_hy_moe_topk_grouped(const float* logits, int64_t ls, int E, int k, const float* corr, int groups,
+                                     int keep, float eps, float* tw, int* te, float* gate, int64_t T, hipStream_t st);
 }
 
 namespace {
@@ -236,19 +263,22 @@ void side_dwa(at::Tensor x, OptT y, OptT sw, double eps, OptT stack, int64_t lay
 }
 
 void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, int64_t dkv_off, OptT dkv_w, double eps,
-                 at::Tensor positions, at::Tensor cos_sin, int64_t dims, at::Tensor cache, at::Tensor slots,
+                 at::Tensor positions, OptT cos_sin, int64_t dims, at::Tensor cache, at::Tensor slots,
                  at::Tensor q_rot, OptT cache_t) {
   rows2d(qgd, "qgd");
   const int f32 = act_f32(qgd);
   same_act(f32, {&cache, &q_rot});
   const int64_t T = qgd.size(0);
-  TORCH_CHECK(H > 0 && dim >= 0 && rd > 0 && R > 0 && dims > 0 && dims % 2 == 0 && dims <= rd &&
-                  H * (dim + rd) <= qgd.size(1), "latent_prep: head sizes");
+  // a model without a rotated part: rd = 0, dims = 0, no table
+  TORCH_CHECK(H > 0 && dim >= 0 && rd >= 0 && dim + rd > 0 && R > 0 && dims >= 0 && dims % 2 == 0 && dims <= rd &&
+                  (dims > 0) == (rd > 0) && H * (dim + rd) <= qgd.size(1), "latent_prep: head sizes");
+  TORCH_CHECK(cos_sin.has_value() == (dims > 0), "latent_prep: a rotation table comes with rot dims, and only then");
   TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
                   positions.numel() == T && slots.is_cuda() && slots.scalar_type() == at::kLong &&
                   slots.is_contiguous() && slots.numel() == T, "latent_prep: positions / slots int64 [T]");
-  TORCH_CHECK(cos_sin.is_cuda() && cos_sin.scalar_type() == at::kFloat && cos_sin.is_contiguous() &&
-                  cos_sin.dim() == 2 && cos_sin.size(1) == dims, "latent_prep: cos_sin fp32 [positions, dims]");
+  if (dims > 0)
+    TORCH_CHECK(cos_sin->is_cuda() && cos_sin->scalar_type() == at::kFloat && cos_sin->is_contiguous() &&
+                    cos_sin->dim() == 2 && cos_sin->size(1) == dims, "latent_prep: cos_sin fp32 [positions, dims]");
   TORCH_CHECK(q_rot.is_contiguous() && q_rot.dim() == 3 && q_rot.size(0) == T && q_rot.size(1) == H &&
                   q_rot.size(2) == rd, "latent_prep: q_rot [T, H, rot_dim]");
   TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd, "latent_prep: cache [pages, page, "
@@ -268,7 +298,8 @@ void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, 
     wp = dkv_w->data_ptr();
   }
   HY_HIP(kafka_hy_latent_prep(f32, qgd.data_ptr(), qgd.stride(0), (int)T, (int)H, (int)dim, (int)rd, (int)R,
-                              (int)dkv_off, wp, (float)eps, positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(),
+                              (int)dkv_off, wp, (float)eps, positions.data_ptr<int64_t>(),
+                              dims > 0 ? cos_sin->data_ptr<float>() : nullptr,
                               (int)dims, cache.data_ptr(), ctp, (int)cache.size(1), slots.data_ptr<int64_t>(),
                               q_rot.data_ptr(), stream()));
 }
@@ -285,8 +316,15 @@ void sigmoid_mul(at::Tensor a, at::Tensor g, at::Tensor out) {
                               (int)H, (int)vd, stream()));
 }
 
+const float* sink_ptr(const OptT& sink, int64_t H) {
+  if (!sink.has_value()) return nullptr;
+  TORCH_CHECK(sink->is_cuda() && sink->scalar_type() == at::kFloat && sink->is_contiguous() && sink->numel() == H,
+              "sink: fp32 [heads]");
+  return sink->data_ptr<float>();
+}
+
 void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tensor bt, at::Tensor tok_seg,
-                 at::Tensor positions, double scale, at::Tensor out) {
+                 at::Tensor positions, double scale, at::Tensor out, int64_t window, OptT sink) {
   const int f32 = act_f32(q_lat);
   same_act(f32, {&q_rot, &cache, &out});
   TORCH_CHECK(q_lat.dim() == 3 && q_lat.stride(2) == 1 && out.dim() == 3 && out.stride(2) == 1 && q_rot.dim() == 3 &&
@@ -295,6 +333,7 @@ void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tenso
   TORCH_CHECK(q_rot.size(0) == T && q_rot.size(1) == H && out.size(0) == H && out.size(1) == T && out.size(2) == R,
               "latent_attn: shapes");
   TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + rd, "latent_attn: cache row");
+  TORCH_CHECK(window >= 0, "latent_attn: window");
   TORCH_CHECK(R + rd <= kafka_hy_latent_attn_max_dk(), "latent_attn: kv_rank + rot_dim beyond ",
               kafka_hy_latent_attn_max_dk());
   TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 &&
@@ -305,14 +344,14 @@ void latent_attn(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tenso
                               q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), (int)cache.size(1), (int)R, (int)rd,
                               bt.data_ptr<int>(), (int)bt.stride(0), tok_seg.data_ptr<int>(),
                               positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(), out.stride(0), out.stride(1),
-                              (int)T, (int)H, stream()));
+                              (int)T, (int)H, (int)window, sink_ptr(sink, H), stream()));
 }
 
 // the matrix-core kernel: items int32 [n, 4] = (first row, tokens, segment, 0), each at most 32 (token, head) rows of
 // one segment (or one token, whose heads go 32 at a time over grid.y)
 void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::Tensor cache_t, at::Tensor bt,
                       at::Tensor items, int64_t tile_tokens, at::Tensor positions, double scale, at::Tensor out,
-                      int64_t nsplit, OptT po, OptT pml) {
+                      int64_t nsplit, OptT po, OptT pml, int64_t window, OptT sink) {
   for (const at::Tensor* t : {&q_lat, &q_rot, &cache, &cache_t, &out})
     TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kBFloat16, "latent_attn_mfma: bf16 GPU tensors");
   TORCH_CHECK(q_lat.dim() == 3 && q_lat.stride(2) == 1 && out.dim() == 3 && out.stride(2) == 1 && q_rot.dim() == 3 &&
@@ -325,9 +364,12 @@ void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::
                   cache_t.size(2) == cache.size(1), "latent_attn_mfma: cache [pages, 16, R + rd] and [pages, R, 16]");
   TORCH_CHECK(kafka_hy_latent_mfma_ok((int)cache.size(1), (int)R, (int)rd), "latent_attn_mfma: sizes not supported");
   // 16-byte loads: every row start must be a multiple of 8 elements
-  TORCH_CHECK(q_lat.stride(0) % 8 == 0 && q_lat.stride(1) % 8 == 0 && q_rot.stride(0) % 8 == 0 &&
-                  q_rot.stride(1) % 8 == 0 && (reinterpret_cast<uintptr_t>(q_lat.data_ptr()) & 15) == 0 &&
-                  (reinterpret_cast<uintptr_t>(q_rot.data_ptr()) & 15) == 0, "latent_attn_mfma: query alignment");
+  TORCH_CHECK(q_lat.stride(0) % 8 == 0 && q_lat.stride(1) % 8 == 0 &&
+                  (reinterpret_cast<uintptr_t>(q_lat.data_ptr()) & 15) == 0, "latent_attn_mfma: query alignment");
+  TORCH_CHECK(rd == 0 || (q_rot.stride(0) % 8 == 0 && q_rot.stride(1) % 8 == 0 &&
+                          (reinterpret_cast<uintptr_t>(q_rot.data_ptr()) & 15) == 0),
+              "latent_attn_mfma: rotated query alignment");
+  TORCH_CHECK(window >= 0, "latent_attn_mfma: window");
   TORCH_CHECK(tile_tokens >= 1 && tile_tokens * std::min<int64_t>(H, 32) <= 32 && (H <= 32 || tile_tokens == 1),
               "latent_attn_mfma: a tile holds at most 32 (token, head) rows");
   TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 && items.is_cuda() &&
@@ -347,7 +389,8 @@ void latent_attn_mfma(at::Tensor q_lat, at::Tensor q_rot, at::Tensor cache, at::
                                    q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), cache_t.data_ptr(), (int)R,
                                    (int)rd, bt.data_ptr<int>(), (int)bt.stride(0), items.data_ptr<int>(),
                                    (int)items.size(0), positions.data_ptr<int64_t>(), (float)scale, out.data_ptr(),
-                                   out.stride(0), out.stride(1), (int)H, (int)nsplit, pop, pmlp, (int)T, stream()));
+                                   out.stride(0), out.stride(1), (int)H, (int)nsplit, pop, pmlp, (int)T, (int)window,
+                                   sink_ptr(sink, H), stream()));
 }
 
 void short_conv(at::Tensor proj, int64_t c0, at::Tensor w, OptT b, at::Tensor tok_seg, at::Tensor seg,
@@ -616,7 +659,8 @@ void moe_topk(at::Tensor logits, at::Tensor tw, at::Tensor te) {
                            te.data_ptr<int>(), T, stream()));
 }
 
-void moe_rows(at::Tensor h, at::Tensor wgu, at::Tensor wd, at::Tensor tw, at::Tensor te, at::Tensor a, at::Tensor out) {
+void moe_rows(at::Tensor h, at::Tensor wgu, at::Tensor wd, at::Tensor tw, at::Tensor te, at::Tensor a, at::Tensor out,
+              double limit, double alpha) {
   rows2d(h, "h"); rows2d(out, "out"); f32t(out, "out"); f32t(tw, "weights");
   const int f32 = act_f32(h);
   same_act(f32, {&wgu, &wd, &a});
@@ -635,7 +679,7 @@ void moe_rows(at::Tensor h, at::Tensor wgu, at::Tensor wd, at::Tensor tw, at::Te
   // expert ids index the weight stacks on the device: the router kernel writes ids in [0, E) only
   HY_HIP(kafka_hy_moe_rows(f32, h.data_ptr(), h.stride(0), wgu.data_ptr(), wd.data_ptr(), tw.data_ptr<float>(),
                            te.data_ptr<int>(), (int)d, (int)F, (int)k, a.data_ptr(), out.data_ptr<float>(),
-                           out.stride(0), T, stream()));
+                           out.stride(0), T, (float)limit, (float)alpha, stream()));
 }
 
 void add2(at::Tensor x, at::Tensor y1, OptT y2, OptT w, double eps, OptT out) {
@@ -662,6 +706,152 @@ void add2(at::Tensor x, at::Tensor y1, OptT y2, OptT w, double eps, OptT out) {
                        (float)eps, op, os, stream()));
 }
 
+// ---- residual streams, windowed attention, group-limited router ---------------------------------------------------
+const float* f32vec(const OptT& t, int64_t n, const char* name) {
+  if (!t.has_value()) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->numel() == n, name,
+              ": fp32 GPU tensor of ", n, " elements expected");
+  return t->data_ptr<float>();
+}
+
+void stream_step(at::Tensor xs, OptT y, OptT mix, OptT write, OptT read, OptT norm_w, double eps, OptT out, OptT y2,
+                 OptT row_scale, OptT total) {
+  TORCH_CHECK(xs.is_cuda() && xs.scalar_type() == at::kFloat && xs.dim() == 3 && xs.stride(2) == 1,
+              "stream_step: streams fp32 [S, T, d] with contiguous rows");
+  const int64_t S = xs.size(0), T = xs.size(1), d = xs.size(2);
+  TORCH_CHECK(S >= 1 && S <= kafka_hy_stream_max(), "stream_step: 1..", kafka_hy_stream_max(), " streams");
+  TORCH_CHECK(T == 0 || (xs.stride(1) >= d && (S == 1 || xs.stride(0) >= d)), "stream_step: overlapping rows");
+  TORCH_CHECK(mix.has_value() == write.has_value() && (!mix.has_value() || y.has_value()),
+              "stream_step: a write needs mix, write and y");
+  TORCH_CHECK(y2.has_value() == row_scale.has_value() && (!y2.has_value() || mix.has_value()),
+              "stream_step: y2 and row_scale come together, with a write");
+  TORCH_CHECK(read.has_value() == norm_w.has_value() && read.has_value() == out.has_value(),
+              "stream_step: a read needs read, norm_w and out");
+  const void *yp = nullptr, *y2p = nullptr;
+  int64_t ys = 0, y2s = 0;
+  int yf = 0, y2f = 0;
+  if (mix.has_value()) {
+    rows2d(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == d, "stream_step: y [T, d]");
+    yp = y->data_ptr(); ys = y->stride(0); yf = act_f32(*y);
+    if (y2.has_value()) {
+      rows2d(*y2, "y2");
+      TORCH_CHECK(y2->size(0) == T && y2->size(1) == d, "stream_step: y2 [T, d]");
+      y2p = y2->data_ptr(); y2s = y2->stride(0); y2f = act_f32(*y2);
+    }
+  }
+  void* op = nullptr; int64_t os = 0; int of = 0;
+  if (out.has_value()) {
+    rows2d(*out, "out");
+    TORCH_CHECK(out->size(0) == T && out->size(1) == d, "stream_step: out [T, d]");
+    op = out->data_ptr(); os = out->stride(0); of = act_f32(*out);
+  }
+  float* tp = nullptr; int64_t ts = 0;
+  if (total.has_value()) {
+    rows2d(*total, "total"); f32t(*total, "total");
+    TORCH_CHECK(total->size(0) == T && total->size(1) == d, "stream_step: total [T, d]");
+    tp = total->data_ptr<float>(); ts = total->stride(0);
+  }
+  HY_HIP(kafka_hy_stream_step(xs.data_ptr<float>(), xs.stride(0), xs.stride(1), (int)S, yp, ys, yf, y2p, y2s, y2f,
+                              f32vec(row_scale, T, "row_scale"), f32vec(mix, S * S, "mix"), f32vec(write, S, "write"),
+                              f32vec(read, S, "read"), f32vec(norm_w, d, "norm_w"), (float)eps, op, os, of, tp, ts, T,
+                              (int)d, stream()));
+}
+
+void swish_clamp_mul(at::Tensor gu, double limit, double alpha, at::Tensor out) {
+  rows2d(gu, "gu"); rows2d(out, "out");
+  const int f32 = act_f32(gu);
+  same_act(f32, {&out});
+  const int64_t T = gu.size(0), F = gu.size(1) / 2;
+  TORCH_CHECK(gu.size(1) == 2 * F && out.size(0) == T && out.size(1) == F && limit > 0,
+              "swish_clamp_mul: gu [T, 2 F], out [T, F], a positive limit");
+  HY_HIP(kafka_hy_swish_clamp_mul(f32, gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), T, (int)F,
+                                  (float)limit, (float)alpha, stream()));
+}
+
+void paged_kv(const at::Tensor& kc, const at::Tensor& vt, int64_t Ck, int64_t Cv, const char* who) {
+  TORCH_CHECK(kc.is_contiguous() && kc.dim() == 3 && kc.size(1) == 16 && kc.size(2) == Ck && vt.is_contiguous() &&
+                  vt.dim() == 3 && vt.size(0) == kc.size(0) && vt.size(1) == Cv && vt.size(2) == 16,
+              who, ": keys [pages, 16, G D] and values [pages, G Dv, 16]");
+}
+
+void qk_norm_rope_store(at::Tensor qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, at::Tensor qw, at::Tensor kw,
+                        double eps, at::Tensor positions, OptT cos_sin, int64_t dims, OptT v_first,
+                        int64_t v_first_off, double lam, at::Tensor kc, at::Tensor vt, at::Tensor slots,
+                        at::Tensor q_out) {
+  rows2d(qkv, "qkv"); rows2d(q_out, "q_out");
+  const int f32 = act_f32(qkv);
+  same_act(f32, {&kc, &vt, &q_out});
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && qkv.size(1) >= H * D + G * D + G * Dv &&
+                  q_out.size(0) == T && q_out.size(1) == H * D, "qk_norm_rope_store: head sizes");
+  TORCH_CHECK(dims >= 0 && dims % 2 == 0 && dims <= D && cos_sin.has_value() == (dims > 0),
+              "qk_norm_rope_store: rot dims even, at most the head size, with their table");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T && slots.is_cuda() && slots.scalar_type() == at::kLong &&
+                  slots.is_contiguous() && slots.numel() == T, "qk_norm_rope_store: positions / slots int64 [T]");
+  if (dims > 0)
+    TORCH_CHECK(cos_sin->is_cuda() && cos_sin->scalar_type() == at::kFloat && cos_sin->is_contiguous() &&
+                    cos_sin->dim() == 2 && cos_sin->size(1) == dims, "qk_norm_rope_store: cos_sin fp32 [positions, dims]");
+  paged_kv(kc, vt, G * D, G * Dv, "qk_norm_rope_store");
+  const void* vfp = nullptr; int64_t vfs = 0;
+  if (v_first.has_value()) {
+    rows2d(*v_first, "v_first"); same_act(f32, {&*v_first});
+    TORCH_CHECK(v_first->size(0) == T && v_first_off >= 0 && v_first_off + G * Dv <= v_first->size(1),
+                "qk_norm_rope_store: the earlier layer's value columns");
+    vfp = v_first->data_ptr(); vfs = v_first->stride(0);
+  }
+  // positions index the table's rows and slots the cache on the device: the step plan keeps both in range
+  HY_HIP(kafka_hy_qk_norm_rope_store(f32, qkv.data_ptr(), qkv.stride(0), (int)H, (int)G, (int)D, (int)Dv,
+                                     f32vec(qw, H * D, "q norm weight"), f32vec(kw, G * D, "k norm weight"), (float)eps,
+                                     positions.data_ptr<int64_t>(), dims > 0 ? cos_sin->data_ptr<float>() : nullptr,
+                                     (int)dims, vfp, vfs, (int)v_first_off, (float)lam, kc.data_ptr(), vt.data_ptr(),
+                                     slots.data_ptr<int64_t>(), q_out.data_ptr(), q_out.stride(0), T, stream()));
+}
+
+void window_attn(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor tok_seg, at::Tensor positions,
+                 int64_t H, int64_t G, double scale, int64_t window, OptT sink, at::Tensor out) {
+  rows2d(q, "q"); rows2d(out, "out");
+  const int f32 = act_f32(q);
+  same_act(f32, {&kc, &vt, &out});
+  const int64_t T = q.size(0);
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && q.size(1) % H == 0 && out.size(0) == T && out.size(1) % H == 0,
+              "window_attn: heads");
+  const int64_t D = q.size(1) / H, Dv = out.size(1) / H;
+  paged_kv(kc, vt, G * D, G * Dv, "window_attn");
+  TORCH_CHECK(D <= kafka_hy_window_attn_max_d() && Dv <= kafka_hy_window_attn_max_dv(), "window_attn: head sizes up to ",
+              kafka_hy_window_attn_max_d(), " / ", kafka_hy_window_attn_max_dv());
+  TORCH_CHECK(window >= 0, "window_attn: window");
+  TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 &&
+                  tok_seg.is_cuda() && tok_seg.scalar_type() == at::kInt && tok_seg.is_contiguous() &&
+                  tok_seg.numel() == T && positions.is_cuda() && positions.scalar_type() == at::kLong &&
+                  positions.is_contiguous() && positions.numel() == T, "window_attn: block tables / tok_seg / positions");
+  HY_HIP(kafka_hy_window_attn(f32, q.data_ptr(), q.stride(0), kc.data_ptr(), vt.data_ptr(), bt.data_ptr<int>(),
+                              (int)bt.stride(0), tok_seg.data_ptr<int>(), positions.data_ptr<int64_t>(), (int)H, (int)G,
+                              (int)D, (int)Dv, (float)scale, (int)window, sink_ptr(sink, H), out.data_ptr(),
+                              out.stride(0), T, stream()));
+}
+
+void moe_topk_grouped(at::Tensor logits, int64_t E, at::Tensor corr, int64_t groups, int64_t keep, double eps,
+                      at::Tensor tw, at::Tensor te, OptT gate) {
+  rows2d(logits, "logits"); f32t(logits, "logits"); f32t(tw, "weights");
+  const int64_t T = logits.size(0);
+  TORCH_CHECK(tw.is_contiguous() && tw.dim() == 2 && tw.size(0) == T && te.is_cuda() && te.is_contiguous() &&
+                  te.scalar_type() == at::kInt && te.sizes() == tw.sizes(), "moe_topk_grouped: outputs [T, k]");
+  const int64_t k = tw.size(1);
+  TORCH_CHECK(E >= 1 && E + (gate.has_value() ? 1 : 0) <= logits.size(1) && E <= kafka_hy_grouped_router_max_e() &&
+                  k >= 1 && k <= kafka_hy_grouped_router_max_k() && groups >= 1 &&
+                  groups <= kafka_hy_grouped_router_max_g() && E % groups == 0 && keep >= 1 && keep <= groups &&
+                  k <= keep * (E / groups),
+              "moe_topk_grouped: up to ", kafka_hy_grouped_router_max_e(), " experts in up to ",
+              kafka_hy_grouped_router_max_g(), " equal groups, ", kafka_hy_grouped_router_max_k(),
+              " per row within the kept groups");
+  HY_HIP(kafka_hy_moe_topk_grouped(logits.data_ptr<float>(), logits.stride(0), (int)E, (int)k,
+                                   f32vec(corr, E, "correction"), (int)groups, (int)keep, (float)eps,
+                                   tw.data_ptr<float>(), te.data_ptr<int>(),
+                                   const_cast<float*>(f32vec(gate, T, "gate")), T, stream()));
+}
+
 }  // namespace
 
 
@@ -682,10 +872,12 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_latent_attn_mfma", &latent_attn_mfma, py::arg("q_lat"), py::arg("q_rot"), py::arg("cache"),
         py::arg("cache_t"), py::arg("bt"), py::arg("items"), py::arg("tile_tokens"), py::arg("positions"),
         py::arg("scale"), py::arg("out"), py::arg("nsplit") = 1, py::arg("po") = py::none(),
-        py::arg("pml") = py::none());
+        py::arg("pml") = py::none(), py::arg("window") = 0, py::arg("sink") = py::none());
   m.def("hy_latent_mfma_ok", [](int page, int R, int rd) { return kafka_hy_latent_mfma_ok(page, R, rd) != 0; });
   m.def("hy_sigmoid_mul", &sigmoid_mul);
-  m.def("hy_latent_attn", &latent_attn);
+  m.def("hy_latent_attn", &latent_attn, py::arg("q_lat"), py::arg("q_rot"), py::arg("cache"), py::arg("bt"),
+        py::arg("tok_seg"), py::arg("positions"), py::arg("scale"), py::arg("out"), py::arg("window") = 0,
+        py::arg("sink") = py::none());
   m.def("hy_short_conv", &short_conv);
   m.def("hy_ssm_scan", &ssm_scan);
   m.def("hy_ssm_combine", &ssm_combine);
@@ -699,9 +891,18 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_mlstm_scan", &mlstm_scan);
   m.def("hy_head_norm_gate", &head_norm_gate);
   m.def("hy_moe_topk", &moe_topk);
-  m.def("hy_moe_rows", &moe_rows);
+  m.def("hy_moe_rows", &moe_rows, py::arg("h"), py::arg("wgu"), py::arg("wd"), py::arg("tw"), py::arg("te"),
+        py::arg("a"), py::arg("out"), py::arg("limit") = 0.0, py::arg("alpha") = 1.0);
   m.def("hy_add2", &add2, py::arg("x"), py::arg("y1"), py::arg("y2") = py::none(), py::arg("w") = py::none(),
         py::arg("eps") = 0.0, py::arg("out") = py::none());
+  m.def("hy_stream_step", &stream_step, py::arg("xs"), py::arg("y") = py::none(), py::arg("mix") = py::none(),
+        py::arg("write") = py::none(), py::arg("read") = py::none(), py::arg("norm_w") = py::none(),
+        py::arg("eps") = 0.0, py::arg("out") = py::none(), py::arg("y2") = py::none(),
+        py::arg("row_scale") = py::none(), py::arg("total") = py::none());
+  m.def("hy_swish_clamp_mul", &swish_clamp_mul);
+  m.def("hy_qk_norm_rope_store", &qk_norm_rope_store);
+  m.def("hy_window_attn", &window_attn);
+  m.def("hy_moe_topk_grouped", &moe_topk_grouped);
   m.def("hy_sigmoid_attn_mfma_ok",
         [](int page, int D, int Dv, int rep) { return kafka_hy_sigmoid_attn_mfma_ok(page, D, Dv, rep) != 0; });
   m.def("hy_sigmoid_attn_mfma", &sigmoid_attn_mfma, py::arg("q"), py::arg("q_off"), py::arg("kc"), py::arg("vt"),

@@ -679,11 +679,23 @@ __global__ __launch_bounds__(NT) void moe_topk_kernel(const float* __restrict__ 
 
 constexpr int MOE_MAXD = 8192;  // the row sits in LDS as fp32
 
-// a[pair][f] = silu(W_gate[e] h) * (W_up[e] h): one workgroup per (pair, block of FB rows), one wave per row
+// a[pair][f] = act(W_gate[e] h, W_up[e] h): one workgroup per (pair, block of FB rows), one wave per row.
+// act(g, u) = silu(g) u, or with limit > 0 the clamped form g' sigmoid(alpha g') (u' + 1), g' = min(g, limit),
+// u' = clamp(u, -limit, limit).
+__device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
 template <typename AT>
 __global__ __launch_bounds__(NT) void moe_gate_up_kernel(const AT* __restrict__ h, int64_t hs,
                                                          const AT* __restrict__ wgu, const int* __restrict__ te, int d,
-                                                         int F, int k, int FB, AT* __restrict__ a) {
+                                                         int F, int k, int FB, AT* __restrict__ a, float limit,
+                                                         float alpha) {
   extern __shared__ float hsh[];
   const int64_t pair = blockIdx.x;
   const int64_t t = pair / k;
@@ -704,7 +716,7 @@ __global__ __launch_bounds__(NT) void moe_gate_up_kernel(const AT* __restrict__ 
     }
     sg = wave_sum(sg);
     su = wave_sum(su);
-    if (lane == 0) stf(a + pair * F + f, sg / (1.0f + expf(-sg)) * su);
+    if (lane == 0) stf(a + pair * F + f, glu_act(sg, su, limit, alpha));
   }
 }
 
@@ -946,7 +958,7 @@ int kafka_hy_moe_rows_max_d() { return MOE_MAXD; }
 
 hipError_t kafka_hy_moe_rows(int f32, const void* h, int64_t hs, const void* wgu, const void* wd, const float* tw,
                              const int* te, int d, int F, int k, void* a, float* out, int64_t os, int64_t T,
-                             hipStream_t st) {
+                             float limit, float alpha, hipStream_t st) {
   if (T <= 0) return hipSuccess;
   if (d > MOE_MAXD || F > MOE_MAXD) return hipErrorInvalidValue;
   // enough workgroups for a step of few rows, many rows per workgroup for a step of many; the down kernel keeps a
@@ -957,7 +969,8 @@ hipError_t kafka_hy_moe_rows(int f32, const void* h, int64_t hs, const void* wgu
   while (T * ((d + cb - 1) / cb) < 1024 && cb > 8) cb = (cb + 1) / 2;
   const dim3 g1((unsigned)pairs, (F + fb - 1) / fb), g2((unsigned)T, (d + cb - 1) / cb);
   DISPATCH_AT(f32, {
-    moe_gate_up_kernel<AT><<<g1, NT, d * sizeof(float), st>>>((const AT*)h, hs, (const AT*)wgu, te, d, F, k, fb, (AT*)a);
+    moe_gate_up_kernel<AT><<<g1, NT, d * sizeof(float), st>>>((const AT*)h, hs, (const AT*)wgu, te, d, F, k, fb, (AT*)a,
+                                                              limit, alpha);
     moe_down_kernel<AT><<<g2, NT, (size_t)F * sizeof(float), st>>>((const AT*)a, (const AT*)wd, tw, te, d, F, k, cb,
                                                                        out, os);
   });

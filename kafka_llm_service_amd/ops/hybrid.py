@@ -75,6 +75,8 @@ def latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot
     """RMS norm of the latent and rotary on the shared key part of the fused projection row -> the row's cache slot
     ([latent | rotated key]; with ``cache_t`` [pages, kv_rank, page] also the latent page-wise transposed, the value
     operand of the matrix-core attention kernel); rotary on every head's query part -> ``q_rot``."""
+    if rd == 0 and (rot_dims or cos_sin is not None):
+        raise ValueError("latent_prep: a rotation needs a rotated part")
     if _gpu(qgd):
         ext().hy_latent_prep(qgd, int(H), int(dim), int(rd), int(R), int(dkv_off), dkv_w, float(eps), positions,
                              cos_sin, int(rot_dims), cache, slot_mapping, q_rot, cache_t)
@@ -116,27 +118,34 @@ def attn_splits(n_tiles: int, heads: int, max_keys: int) -> int:
 
 
 def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out, cache_t=None,
-                tiles=None, max_keys: int = 0) -> None:
+                tiles=None, max_keys: int = 0, window: int = 0, sink=None) -> None:
     """Causal softmax attention of every row's heads over its sequence's cached [latent | rotated key] rows:
     out[h, t] = sum_j softmax_j((q_lat[h, t] . c_j + q_rot[t, h] . k_j) scale) c_j over the keys j <= position[t].
     With the transposed latent copy ``cache_t`` and ``tiles`` (int32 [n, 4] = (first row, tokens, segment, 0), at
     most ``tile_tokens(H)`` tokens of one segment each) bf16 runs on the matrix cores; else one wave per (row, 4
     heads) on the vector units (fp32, odd sizes). ``max_keys`` (the step's longest context) lets a launch of few
-    tiles split its key ranges over more workgroups (``attn_splits``)."""
+    tiles split its key ranges over more workgroups (``attn_splits``).
+    ``window`` > 0: a row at position p sees only the keys p - window < j <= p. ``sink`` fp32 [H]: a per-head logit
+    (not scaled) that joins the softmax denominator without a key or a value."""
+    if window < 0:
+        raise ValueError("latent_attn: window must be positive (0 = every earlier position)")
     if _gpu(q_lat):
         if cache_t is not None and tiles is not None and q_lat.dtype == torch.bfloat16:
             H, T, R = q_lat.shape
+            if window:  # a key range is at most the window long
+                max_keys = min(max_keys, window + tile_tokens(H))
             ns = attn_splits(tiles.shape[0], H, max_keys) if max_keys else 1
             po = pml = None
             if ns > 1:
                 po = torch.empty(ns, H, T, R, dtype=torch.float32, device=q_lat.device)
                 pml = torch.empty(ns, H, T, 2, dtype=torch.float32, device=q_lat.device)
             ext().hy_latent_attn_mfma(q_lat, q_rot, cache, cache_t, block_tables, tiles, tile_tokens(H), positions,
-                                      float(scale), out, ns, po, pml)
+                                      float(scale), out, ns, po, pml, int(window), sink)
         else:
-            ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out)
+            ext().hy_latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, positions, float(scale), out, int(window),
+                                 sink)
     else:
-        ref.latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out)
+        ref.latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out, window, sink)
 
 
 def sigmoid_mul(a, g, out) -> None:
@@ -356,16 +365,32 @@ def moe_router(h, w, b, k: int):
     return tw, te
 
 
-def moe_rows(h, w_gu, w_down, topk_w, topk_e, out) -> None:
+GLU_ACTS = ("silu", "swish_clamp")
+
+
+def _glu_act(act: str, limit: float, alpha: float) -> tuple[float, float]:
+    """(limit, alpha) as the kernels take them: limit 0 selects silu(g) * u."""
+    if act not in GLU_ACTS:
+        raise ValueError(f"unknown gated activation {act!r}")
+    if act == "silu":
+        return 0.0, 1.0
+    if not limit > 0:
+        raise ValueError("swish_clamp needs a positive limit")
+    return float(limit), float(alpha)
+
+
+def moe_rows(h, w_gu, w_down, topk_w, topk_e, out, act: str = "silu", limit: float = 0.0, alpha: float = 1.0) -> None:
     """Routed experts evaluated per (row, chosen expert) pair, any sizes and both dtypes:
-    out[t] = sum_j topk_w[t, j] W_down[e_tj] (silu(W_gate[e_tj] h_t) * W_up[e_tj] h_t) with w_gu [E, 2 F, d] = gate
-    rows then up rows and w_down [E, d, F]; the pairs of a row are summed in order j = 0, 1, ... (fp32)."""
+    out[t] = sum_j topk_w[t, j] W_down[e_tj] act(W_gate[e_tj] h_t, W_up[e_tj] h_t) with w_gu [E, 2 F, d] = gate
+    rows then up rows and w_down [E, d, F]; the pairs of a row are summed in order j = 0, 1, ... (fp32).
+    ``act``: "silu" = silu(g) * u, or "swish_clamp" (see ``swish_clamp_mul``)."""
+    lim, al = _glu_act(act, limit, alpha)
     if _gpu(h):
         T, k = topk_e.shape
         a = torch.empty(T * k, w_down.shape[2], dtype=h.dtype, device=h.device)
-        ext().hy_moe_rows(h, w_gu, w_down, topk_w, topk_e, a, out)
+        ext().hy_moe_rows(h, w_gu, w_down, topk_w, topk_e, a, out, lim, al)
     else:
-        ref.moe_rows(h, w_gu, w_down, topk_w, topk_e, out)
+        ref.moe_rows(h, w_gu, w_down, topk_w, topk_e, out, lim, al)
 
 
 MOE_STREAM_MAX_T = 640  # steps of up to this many rows run tiled expert weights on the grouped streaming kernel
@@ -378,26 +403,33 @@ def moe_grouped_ok(h, w_gu, w_down) -> bool:
                 h.stride(0) % 8 == 0)
 
 
-def moe_experts(h, w_gu, w_down, topk_w, topk_e, out, w_gu_t=None, w_down_t=None) -> None:
+def moe_experts(h, w_gu, w_down, topk_w, topk_e, out, w_gu_t=None, w_down_t=None, act: str = "silu",
+                limit: float = 0.0, alpha: float = 1.0) -> None:
     """out (fp32 [T, d]) = the routed experts' weighted sum for every row. Sizes the framework's expert-sorted
     matrix-core kernels take (bf16) go through them - entries sorted by expert (``ops.moe_sort``), gate/up GEMM on
     gathered rows, silu * up, down GEMM with the weighted combine in its epilogue (fp32 adds, two entries per row
     commute), or the grouped weight-streaming kernels when tiled expert weights are given and the step is small -
-    everything else is evaluated per (row, expert) pair by ``moe_rows``."""
+    everything else is evaluated per (row, expert) pair by ``moe_rows``. ``act`` as in ``moe_rows`` (the streaming
+    kernels have silu built in; another activation runs between the two expert-sorted GEMMs)."""
     from kafka_llm_service_amd import ops
 
     T = h.shape[0]
     if T and moe_grouped_ok(h, w_gu, w_down):
         r = ops.moe_sort(topk_w, topk_e, w_gu.shape[0])
         out.zero_()
-        if w_gu_t is not None and w_down_t is not None and T <= MOE_STREAM_MAX_T:
+        if act == "silu" and w_gu_t is not None and w_down_t is not None and T <= MOE_STREAM_MAX_T:
             a = ops.grouped_stream_glu(h, w_gu_t, r)
             ops.grouped_stream_combine(a, w_down_t, r, T, out)
         else:
-            a = ops.silu_mul(ops.grouped_gemm(h, w_gu, r, gather=True))
+            gu = ops.grouped_gemm(h, w_gu, r, gather=True)
+            if act == "silu":
+                a = ops.silu_mul(gu)
+            else:
+                a = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+                swish_clamp_mul(gu, limit, alpha, a)
             ops.grouped_gemm(a, w_down, r, gather=False, combine_out=out)
     else:
-        moe_rows(h, w_gu, w_down, topk_w, topk_e, out)
+        moe_rows(h, w_gu, w_down, topk_w, topk_e, out, act, limit, alpha)
 
 
 def add2(x, y1, y2=None, norm_w=None, eps=0.0, out=None) -> None:
@@ -409,3 +441,105 @@ def add2(x, y1, y2=None, norm_w=None, eps=0.0, out=None) -> None:
         ref.add2(x, y1, y2)
         if norm_w is not None:
             ref.rms_norm(x, norm_w, eps, out)
+
+
+# ---- hyper-connected residual streams, windowed softmax attention with sinks, group-limited routing -----------------
+STREAM_MAX = 8   # residual streams the stream kernel keeps in registers
+
+
+def stream_step(xs, y=None, mix=None, write=None, read=None, norm_w=None, eps=0.0, out=None, y2=None,
+                row_scale=None, total=None) -> None:
+    """One pass over the residual streams xs fp32 [S, T, d] (hyper-connections), every part optional:
+      write   with ``mix`` fp32 [S, S] (indexed [from, to]) and ``write`` fp32 [S]: all streams at once from the old
+              ones, xs[r] <- sum_s mix[s, r] xs[s] + write[r] * (y + row_scale[:, None] * y2); y / y2 [T, d] in the
+              activation dtype or fp32, row_scale fp32 [T] (y2 and row_scale come together or not at all);
+      read    with ``read`` fp32 [S] and ``norm_w`` fp32 [d] (a one-plus weight is passed as 1 + w): out = u /
+              sqrt(mean(u^2) + eps) * norm_w for u = sum_s read[s] xs[s] of the NEW streams, in out's dtype;
+      total   fp32 [T, d] <- sum_s xs[s] of the new streams.
+    All arithmetic is fp32. A plain residual is S = 1 with mix = write = read = 1."""
+    S = xs.shape[0]
+    if S > STREAM_MAX:
+        raise ValueError(f"stream_step: at most {STREAM_MAX} streams")
+    if (mix is None) != (write is None) or (mix is not None and y is None):
+        raise ValueError("stream_step: a write needs mix, write and y")
+    if (y2 is None) != (row_scale is None) or (y2 is not None and mix is None):
+        raise ValueError("stream_step: y2 and row_scale come together, with a write")
+    if (read is None) != (norm_w is None) or (read is None) != (out is None):
+        raise ValueError("stream_step: a read needs read, norm_w and out")
+    if _gpu(xs):
+        ext().hy_stream_step(xs, y, mix, write, read, norm_w, float(eps), out, y2, row_scale, total)
+    else:
+        ref.stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total)
+
+
+def swish_clamp_mul(gu, limit: float, alpha: float, out) -> None:
+    """out = g' sigmoid(alpha g') (u' + 1) with g' = min(gu[:, :F], limit), u' = clamp(gu[:, F:], -limit, limit)."""
+    if not limit > 0:
+        raise ValueError("swish_clamp_mul needs a positive limit")
+    if _gpu(gu):
+        ext().hy_swish_clamp_mul(gu, float(limit), float(alpha), out)
+    else:
+        ref.swish_clamp_mul(gu, limit, alpha, out)
+
+
+def qk_norm_rope_store(qkv, H: int, G: int, D: int, Dv: int, q_w, k_w, eps, positions, cos_sin, rot_dims: int,
+                       v_first, v_first_off: int, lam: float, k_cache, v_cache_t, slot_mapping, q_out) -> None:
+    """Attention inputs from the fused projection row [q (H D) | k (G D) | v (G Dv)]:
+      * RMS norm over the WHOLE q part and over the whole k part (weights fp32 [H D], [G D]), before the split into heads;
+      * rotation of the dimension pairs (2i, 2i + 1), i < rot_dims / 2, of every q and k head by the row's position
+        (``cos_sin`` fp32 [positions, rot_dims] = cos | sin per frequency; rot_dims = 0 and no table: no rotation);
+      * values: with ``v_first`` (rows [T, ...] whose value columns start at ``v_first_off``) v <- (1 - lam) v + lam
+        v_first;
+      * q -> q_out [T, H D]; k -> k_cache [pages, page, G D] at the row's slot; v -> v_cache_t [pages, G Dv, page].
+    Norms, rotation and the mix are fp32."""
+    if rot_dims % 2 or rot_dims > D or (rot_dims > 0) != (cos_sin is not None):
+        raise ValueError("qk_norm_rope_store: rot_dims even, at most the head size, with its table")
+    if _gpu(qkv):
+        ext().hy_qk_norm_rope_store(qkv, int(H), int(G), int(D), int(Dv), q_w, k_w, float(eps), positions, cos_sin,
+                                    int(rot_dims), v_first, int(v_first_off), float(lam), k_cache, v_cache_t,
+                                    slot_mapping, q_out)
+    else:
+        ref.qk_norm_rope_store(qkv, H, G, D, Dv, q_w, k_w, eps, positions, cos_sin, rot_dims, v_first, v_first_off,
+                               lam, k_cache, v_cache_t, slot_mapping, q_out)
+
+
+def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int, G: int, scale: float, window: int,
+                sink, out) -> None:
+    """Causal softmax attention over paged keys [pages, page, G D] and page-wise transposed values [pages, G Dv, page]:
+    row t at position p, head h (key/value head h // (H / G)) sees the keys p - window < j <= p (window 0: all j <= p);
+        out = sum_j e^(s_j) v_j / (sum_j e^(s_j) + e^(sink[h])),  s_j = (q . k_j) scale
+    with ``sink`` fp32 [H] (None: no such term). q [T, H D], out [T, H Dv]; scores and weights fp32. One wave per
+    (row, head), keys in order, whatever the batch."""
+    if window < 0:
+        raise ValueError("window_attn: window must be positive (0 = every earlier position)")
+    if _gpu(q):
+        ext().hy_window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, int(H), int(G), float(scale),
+                             int(window), sink, out)
+    else:
+        ref.window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out)
+
+
+def moe_router_grouped(h, w, correction, k: int, groups: int, keep: int, eps: float = 0.0, extra_gate: bool = False):
+    """Group-limited router: fp32 logits h W^T over the first E rows of ``w`` (fp32 [E (+ 1), d]); s = softmax over
+    all E; the choice looks at s + correction, only within the ``keep`` groups (of ``groups`` equal groups of
+    neighbouring experts) whose largest corrected score is largest, and takes the k largest there (ties: the lower
+    index); the weights are s of the chosen divided by (their sum + eps). With ``extra_gate`` the last row of ``w`` is
+    a gate vector and sigmoid of its product is returned per row. Returns (weights fp32 [T, k], experts int32
+    [T, k], gate fp32 [T] or None)."""
+    T = h.shape[0]
+    E = w.shape[0] - (1 if extra_gate else 0)
+    if E < 1 or groups < 1 or E % groups or not 1 <= keep <= groups or not 1 <= k <= keep * (E // groups):
+        raise ValueError("router: experts, groups and choices do not fit")
+    if correction.shape[0] != E:
+        raise ValueError("router: one correction per expert")
+    tw = torch.empty(T, k, dtype=torch.float32, device=h.device)
+    te = torch.empty(T, k, dtype=torch.int32, device=h.device)
+    gate = torch.empty(T, dtype=torch.float32, device=h.device) if extra_gate else None
+    if _gpu(h):
+        # logits as one full-precision fp32 matrix product (the engine switches reduced-precision matrix modes off),
+        # then the choice kernel
+        ext().hy_moe_topk_grouped(torch.mm(h.float(), w.t()), int(E), correction, int(groups), int(keep), float(eps),
+                                  tw, te, gate)
+    else:
+        ref.moe_router_grouped(h, w, E, correction, k, groups, keep, eps, tw, te, gate)
+    return tw, te, gate

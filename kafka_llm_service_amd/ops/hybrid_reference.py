@@ -75,7 +75,7 @@ def latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot
     rotated query parts into ``q_rot`` [T, H, rd]."""
     T = qgd.shape[0]
     half = rot_dims // 2
-    cs = cos_sin[positions.long()]
+    cs = cos_sin[positions.long()] if cos_sin is not None else torch.zeros(T, 0)
     c, s = cs[:, :half], cs[:, half:]
 
     def rot(v):  # [T, ..., rd]
@@ -95,8 +95,9 @@ def latent_prep(qgd, H, dim, rd, R, dkv_off, dkv_w, eps, positions, cos_sin, rot
         cache.view(-1, R + rd)[slot_mapping[ok].long()] = row[ok]
 
 
-def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out):
-    """q_lat [H, T, R], q_rot [T, H, rd], cache [pages, page, R + rd]; out [H, T, R] = softmax-weighted latents."""
+def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scale, out, window=0, sink=None):
+    """q_lat [H, T, R], q_rot [T, H, rd], cache [pages, page, R + rd]; out [H, T, R] = softmax-weighted latents over
+    the keys of the row's window (0: all earlier ones); ``sink`` [H] joins the denominator only."""
     H, T, R = q_lat.shape
     page = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1]).float()
@@ -106,8 +107,12 @@ def latent_attn(q_lat, q_rot, cache, block_tables, tok_seg, seg, positions, scal
         pages = block_tables[r, :(n + page - 1) // page].long()
         idx = (pages[:, None] * page + torch.arange(page)[None]).reshape(-1)[:n]
         kv = flat[idx]
+        if window:
+            kv = kv[max(0, n - window):]
         s = (q_lat[:, t].float() @ kv[:, :R].T + q_rot[t].float() @ kv[:, R:].T) * scale
-        out[:, t] = (torch.softmax(s, -1) @ kv[:, :R]).to(out.dtype)
+        if sink is not None:
+            s = torch.cat([s, sink.float()[:, None]], 1)
+        out[:, t] = (torch.softmax(s, -1)[:, :kv.shape[0]] @ kv[:, :R]).to(out.dtype)
 
 
 def sigmoid_mul(a, g, out):
@@ -277,9 +282,17 @@ def moe_router(h, w, b, k, topk_w, topk_e):
     topk_w.copy_(torch.softmax(val[:, :k], -1))
 
 
-def moe_rows(h, w_gu, w_down, topk_w, topk_e, out):
-    """out[t] = sum_j topk_w[t, j] W_down[e] (silu(W_gate[e] h_t) * W_up[e] h_t), e = topk_e[t, j]; w_gu [E, 2 F, d]
-    = gate rows then up rows, w_down [E, d, F]; out in the activation dtype."""
+def _glu(gu, Fh, limit, alpha):
+    g, u = gu[:, :Fh], gu[:, Fh:]
+    if limit > 0:
+        g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+        return g * torch.sigmoid(alpha * g) * (u + 1.0)
+    return F.silu(g) * u
+
+
+def moe_rows(h, w_gu, w_down, topk_w, topk_e, out, limit=0.0, alpha=1.0):
+    """out[t] = sum_j topk_w[t, j] W_down[e] act(W_gate[e] h_t, W_up[e] h_t), e = topk_e[t, j]; w_gu [E, 2 F, d]
+    = gate rows then up rows, w_down [E, d, F]; act = silu(g) * u, or with a limit the clamped swish form."""
     T, k = topk_e.shape
     Fh = w_down.shape[2]
     hf = h.float()
@@ -287,7 +300,7 @@ def moe_rows(h, w_gu, w_down, topk_w, topk_e, out):
     for j in range(k):
         e = topk_e[:, j].long()
         gu = torch.einsum("tfd,td->tf", w_gu[e].float(), hf)
-        a = (F.silu(gu[:, :Fh]) * gu[:, Fh:]).to(h.dtype).float()
+        a = _glu(gu, Fh, limit, alpha).to(h.dtype).float()
         acc += topk_w[:, j:j + 1].float() * torch.einsum("tdf,tf->td", w_down[e].float(), a)
     out.copy_(acc)
 
@@ -296,3 +309,82 @@ def add2(x, y1, y2=None):
     """x += y1 (+ y2), summed in fp32."""
     s = y1.float() if y2 is None else y1.float() + y2.float()
     x += s
+
+
+def stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total):
+    """xs fp32 [S, T, d]: optional write (all streams from the old ones), optional normed read, optional sum."""
+    if mix is not None:
+        ys = y.float()
+        if y2 is not None:
+            ys = ys + row_scale.float()[:, None] * y2.float()
+        new = torch.einsum("sr,std->rtd", mix.float(), xs) + write.float()[:, None, None] * ys[None]
+        xs.copy_(new)
+    if read is not None:
+        u = torch.einsum("s,std->td", read.float(), xs)
+        out.copy_((u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * norm_w.float()).to(out.dtype))
+    if total is not None:
+        total.copy_(xs.sum(0))
+
+
+def swish_clamp_mul(gu, limit, alpha, out):
+    out.copy_(_glu(gu.float(), gu.shape[1] // 2, limit, alpha).to(out.dtype))
+
+
+def qk_norm_rope_store(qkv, H, G, D, Dv, q_w, k_w, eps, positions, cos_sin, rot_dims, v_first, v_first_off, lam,
+                       k_cache, v_cache_t, slot_mapping, q_out):
+    T = qkv.shape[0]
+    Cq, Ck, Cv = H * D, G * D, G * Dv
+    q, k, v = (t.float() for t in qkv[:, :Cq + Ck + Cv].split([Cq, Ck, Cv], 1))
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_w.float()
+    k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_w.float()
+    q, k = q.view(T, H, D).clone(), k.view(T, G, D).clone()
+    if rot_dims:
+        half = rot_dims // 2
+        cs = cos_sin[positions.long()]
+        c, s = cs[:, None, :half], cs[:, None, half:]
+        for x in (q, k):
+            a, b = x[..., 0:rot_dims:2].clone(), x[..., 1:rot_dims:2].clone()
+            x[..., 0:rot_dims:2] = a * c - b * s
+            x[..., 1:rot_dims:2] = b * c + a * s
+    if v_first is not None:
+        v = (1.0 - lam) * v + lam * v_first[:, v_first_off:v_first_off + Cv].float()
+    q_out.copy_(q.reshape(T, Cq).to(q_out.dtype))
+    kv_store(torch.cat([k.reshape(T, Ck), v], 1).to(k_cache.dtype), 0, Ck, k_cache, v_cache_t, slot_mapping)
+
+
+def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out):
+    T = q.shape[0]
+    page, D = k_cache.shape[1], k_cache.shape[2] // G
+    Dv = v_cache_t.shape[1] // G
+    rep = H // G
+    for t in range(T):
+        r, n = int(tok_seg[t]), int(positions[t]) + 1
+        pages = block_tables[r, :(n + page - 1) // page].long()
+        lo = max(0, n - window) if window else 0
+        k = k_cache[pages].reshape(-1, G, D)[lo:n].float()                       # [n, G, D]
+        v = v_cache_t[pages].permute(0, 2, 1).reshape(-1, G, Dv)[lo:n].float()   # [n, G, Dv]
+        qt = q[t].float().view(H, D)
+        s = torch.einsum("hd,jhd->hj", qt, k.repeat_interleave(rep, 1)) * scale
+        if sink is not None:
+            s = torch.cat([s, sink.float()[:, None]], 1)
+        pw = torch.softmax(s, -1)[:, :n - lo]
+        out[t] = torch.einsum("hj,jhv->hv", pw, v.repeat_interleave(rep, 1)).reshape(H * Dv).to(out.dtype)
+
+
+def moe_router_grouped(h, w, E, correction, k, groups, keep, eps, topk_w, topk_e, gate):
+    z = h.float() @ w.float().T
+    s = torch.softmax(z[:, :E], -1)
+    choice = s + correction.float()
+    T = h.shape[0]
+    gsz = E // groups
+    gs = choice.view(T, groups, gsz).max(-1).values
+    gi = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+    ok = torch.zeros(T, groups, dtype=torch.bool)
+    ok.scatter_(1, gi, True)
+    choice = choice.masked_fill(~ok[:, :, None].expand(T, groups, gsz).reshape(T, E), float("-inf"))
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :k]
+    wv = s.gather(1, idx)
+    topk_e.copy_(idx)
+    topk_w.copy_(wv / (wv.sum(-1, keepdim=True) + eps))
+    if gate is not None:
+        gate.copy_(torch.sigmoid(z[:, E]))

@@ -57,32 +57,45 @@ def attention_values(h, W, p):
     return h @ W[p + "v"].T + W[p + "v.b"]
 
 
-def attention(h, W, p, m, eps, v_first=None):
-    """Grouped-query attention with whole-projection query / key norms, pairwise rotation, a sliding window and a
-    sink. ``v_first``: the values of the first value-mixing layer when this is a later one."""
-    T = h.shape[0]
-    H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
-    q = h @ W[p + "q"].T + W[p + "q.b"]
-    k = h @ W[p + "k"].T + W[p + "k.b"]
-    v = attention_values(h, W, p)
-    q = rms_unit(q, eps) * W[p + "q.norm"]
-    k = rms_unit(k, eps) * W[p + "k.norm"]
-    q, k = q.view(T, H, D), k.view(T, G, D)
+def attention_inputs(q, k, qw, kw, m, eps):
+    """q [T, H D], k [T, G D] as projected -> (q [T, H, D], k [T, G, D]): RMS norm over each whole projection with
+    its plain weight, split into heads, pairwise rotation."""
+    T = q.shape[0]
+    H, G, D = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
+    q = (rms_unit(q, eps) * qw).view(T, H, D)
+    k = (rms_unit(k, eps) * kw).view(T, G, D)
     rot = m.get("rot")
     if rot:
         q = rotate_pairs(q, int(rot["dims"]), float(rot["base"]))
         k = rotate_pairs(k, int(rot["dims"]), float(rot["base"]))
+    return q, k
+
+
+def windowed_attention(q, k, v, scale, window, sink):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv] (query head h reads key/value head h // (H / G)) -> [T, H Dv]."""
+    T, H = q.shape[0], q.shape[1]
+    rep = H // k.shape[1]
+    kh = k.repeat_interleave(rep, 1).permute(1, 0, 2)
+    vh = v.repeat_interleave(rep, 1).permute(1, 0, 2)
+    s = torch.einsum("thd,hjd->htj", q, kh) * float(scale)
+    pw = sink_softmax(s, visible(T, window), sink)
+    return torch.einsum("htj,hjv->thv", pw, vh).reshape(T, -1)
+
+
+def attention(h, W, p, m, eps, v_first=None):
+    """Grouped-query attention with whole-projection query / key norms, pairwise rotation, a sliding window and a
+    sink. ``v_first``: the values of the first value-mixing layer when this is a later one."""
+    T = h.shape[0]
+    G, Dv = int(m["kv_heads"]), int(m["vdim"])
+    q = h @ W[p + "q"].T + W[p + "q.b"]
+    k = h @ W[p + "k"].T + W[p + "k.b"]
+    v = attention_values(h, W, p)
+    q, k = attention_inputs(q, k, W[p + "q.norm"], W[p + "k.norm"], m, eps)
     if v_first is not None:
         lam = W[p + "vmix"]
         v = (1.0 - lam) * v + lam * v_first
-    v = v.view(T, G, Dv)
-    rep = H // G
-    kh = k.repeat_interleave(rep, 1).permute(1, 0, 2)
-    vh = v.repeat_interleave(rep, 1).permute(1, 0, 2)
-    s = torch.einsum("thd,hjd->htj", q, kh) * float(m["scale"])
     win = (m.get("mask") or {}).get("size")
-    pw = sink_softmax(s, visible(T, win), W[p + "sink"])
-    o = torch.einsum("htj,hjv->thv", pw, vh).reshape(T, H * Dv)
+    o = windowed_attention(q, k, v.view(T, G, Dv), m["scale"], win, W[p + "sink"])
     return o @ W[p + "o"].T
 
 
@@ -94,30 +107,27 @@ def latent_attention(h, W, p, m, eps):
     c = rms_unit(h @ W[p + "dkv"].T, eps) * W[p + "dkv.norm"]
     k = (c @ W[p + "uk"].T).view(T, H, D)
     v = (c @ W[p + "uv"].T).view(T, H, Dv)
-    s = torch.einsum("thd,jhd->htj", q, k) * float(m["scale"])
     win = (m.get("mask") or {}).get("size")
-    pw = sink_softmax(s, visible(T, win), W[p + "sink"])
-    o = torch.einsum("htj,jhv->thv", pw, v).reshape(T, H * Dv)
+    o = windowed_attention(q, k, v, m["scale"], win, W[p + "sink"])
     return o @ W[p + "o"].T
+
+
+def swish_clamp(g, u, limit, alpha=1.702):
+    g = g.clamp(max=limit)
+    u = u.clamp(min=-limit, max=limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1.0)
 
 
 def expert(h, W, p, limit):
     """Clamped gated unit: gate capped from above, up clamped both ways, gate * sigmoid(1.702 gate) * (up + 1)."""
-    g = (h @ W[p + "gate"].T).clamp(max=limit)
-    u = (h @ W[p + "up"].T).clamp(min=-limit, max=limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ W[p + "down"].T
+    return swish_clamp(h @ W[p + "gate"].T, h @ W[p + "up"].T, limit) @ W[p + "down"].T
 
 
-def route(h, W, p, mlp):
-    """(weights [T, top], experts [T, top]): softmax over all experts; the choice adds the correction and keeps only
-    the best groups; the weights are the uncorrected scores of the chosen, normalised."""
-    r = mlp["router"]
-    E, top = int(r["experts"]), int(r["top"])
-    gr = r.get("groups") or {}
-    n_g, keep = int(gr.get("count", 1)), int(gr.get("keep", 1))
-    s = torch.softmax(h @ W[p + "router"].T, -1)
-    choice = s + W[p + "correction"]
-    T = h.shape[0]
+def route_logits(z, correction, top, n_g, keep):
+    """Router logits z [T, E] -> (weights [T, top], experts [T, top])."""
+    T, E = z.shape
+    s = torch.softmax(z, -1)
+    choice = s + correction
     gs = choice.view(T, n_g, E // n_g).max(-1).values
     best = gs.topk(keep, -1).indices
     allowed = torch.zeros(T, n_g, dtype=torch.bool)
@@ -126,6 +136,15 @@ def route(h, W, p, mlp):
     idx = choice.masked_fill(~allowed, float("-inf")).topk(top, -1).indices
     w = s.gather(1, idx)
     return w / (w.sum(-1, keepdim=True) + 1e-20), idx
+
+
+def route(h, W, p, mlp):
+    """(weights [T, top], experts [T, top]): softmax over all experts; the choice adds the correction and keeps only
+    the best groups; the weights are the uncorrected scores of the chosen, normalised."""
+    r = mlp["router"]
+    gr = r.get("groups") or {}
+    return route_logits(h @ W[p + "router"].T, W[p + "correction"], int(r["top"]), int(gr.get("count", 1)),
+                        int(gr.get("keep", 1)))
 
 
 def feed_forward(h, W, p, mlp):

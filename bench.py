@@ -105,7 +105,9 @@ def parse(argv=None):
                     help="decode measurements as <sequences>x<context tokens>")
     ap.add_argument("--arch-models", default="budurax,llama",
                     help="model families to measure, of budurax, llama, lisorax (sigmoid attention, rglru, mlstm "
-                         "layers with 8 routed experts, 2 per token, of half the dense feed-forward each)")
+                         "layers with 8 routed experts, 2 per token, of half the dense feed-forward each), mozidra "
+                         "(windowed latent and grouped-query attention over 4 residual streams; 8 group-routed "
+                         "experts, 2 per token, and a shared one, of a third of the dense feed-forward each)")
     return ap.parse_args(argv)
 
 
@@ -116,9 +118,10 @@ def arch_compare(args) -> int:
     import torch
 
     from kafka_llm_service_amd.engine.engine import EngineConfig, LLMEngine
-    from kafka_llm_service_amd.models.config import ModelConfig, _budurax, _lisorax
+    from kafka_llm_service_amd.models.config import ModelConfig, _budurax, _lisorax, _mozidra
     from kafka_llm_service_amd.models.budurax import BuduraxConfig
     from kafka_llm_service_amd.models.lisorax import LisoraxConfig
+    from kafka_llm_service_amd.models.mozidra import MozidraConfig
 
     dev = "cuda:0" if torch.cuda.is_available() else "cpu"
     w, L = args.arch_width, args.arch_layers
@@ -129,6 +132,8 @@ def arch_compare(args) -> int:
     cfgs = {"budurax": BuduraxConfig.from_dict(_budurax(w, heads, L, vocab, ff), name=f"budurax-w{w}-l{L}"),
             "lisorax": LisoraxConfig.from_dict(_lisorax(w, heads, max(1, heads // 4), L, vocab, ff // 2 // 256 * 256),
                                                name=f"lisorax-w{w}-l{L}"),
+            "mozidra": MozidraConfig.from_dict(_mozidra(w, heads, max(1, heads // 4), L, vocab, ff // 3 // 256 * 256),
+                                               name=f"mozidra-w{w}-l{L}"),
             "llama": ModelConfig(name=f"llama-w{w}-l{L}", hidden_size=w, intermediate_size=ff, num_layers=L,
                                  num_heads=heads, num_kv_heads=max(1, heads // 4), vocab_size=vocab,
                                  max_position_embeddings=131072, bos_token_id=1, eos_token_ids=[2])}

@@ -384,6 +384,10 @@ class MozidraLM:
             else:
                 lw.z = None
             self.layers.append(lw)
+        # tile sizes (tokens) the step plan must carry for the matrix-core attention kernels
+        self.attn_tile_tokens = sorted({hops.tile_tokens(int(lw.m["heads"])) if lw.type == "latent_attention" else
+                                        hops.sig_tile_tokens(int(lw.m["heads"]), int(lw.m["kv_heads"]))
+                                        for lw in self.layers})
         return self
 
     def _rot_table(self, rot: dict) -> torch.Tensor:
@@ -402,8 +406,8 @@ class MozidraLM:
             m = L["mixer"]
             if L["type"] == "attention":
                 n += int(m["kv_heads"]) * (int(m["dim"]) + int(m["vdim"]))
-            else:
-                n += int(m["kv_rank"])
+            else:  # (the latent is kept twice where the matrix-core kernel runs: row-major and page-wise transposed)
+                n += 2 * int(m["kv_rank"])
         return PAGE * n * es or 1
 
     def alloc_cache(self, num_blocks: int, num_slots: int):
@@ -412,14 +416,19 @@ class MozidraLM:
         patterns for the debug checks."""
         dev, dt = self.device, self.dtype
         pages = []
+        self.pages_t = []  # page-wise transposed latent copies [blocks, kv_rank, 16] where the matrix-core kernel applies
         for lw in self.layers:
             m = lw.m
             if lw.type == "attention":
                 G, D, Dv = (int(m[k]) for k in ("kv_heads", "dim", "vdim"))
                 pages.append((torch.zeros(num_blocks, PAGE, G * D, dtype=dt, device=dev),
                               torch.zeros(num_blocks, G * Dv, PAGE, dtype=dt, device=dev)))
+                self.pages_t.append(None)
             else:
-                pages.append(torch.zeros(num_blocks, PAGE, int(m["kv_rank"]), dtype=dt, device=dev))
+                R = int(m["kv_rank"])
+                pages.append(torch.zeros(num_blocks, PAGE, R, dtype=dt, device=dev))
+                self.pages_t.append(torch.zeros(num_blocks, R, PAGE, dtype=dt, device=dev)
+                                    if hops.latent_mfma_ok(pages[-1], R, 0) else None)
         return pages, PageState()
 
     # one step ---------------------------------------------------------------------------------------------------
@@ -474,7 +483,7 @@ class MozidraLM:
             step[i] = (qkv, H * D + G * D)
         ao = torch.empty(T, H * Dv, dtype=dt, device=dev)
         hops.window_attn(q, k_cache, v_cache_t, m.block_tables, m.tok_seg, inp.positions, H, G, lw.scale, lw.window,
-                         lw.sink, ao)
+                         lw.sink, ao, m.tiles.get(hops.sig_tile_tokens(H, G)), m.max_keys)
         return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 
     def _latent_attention(self, i: int, lw, h, inp, m: SegMeta, pages: list) -> torch.Tensor:
@@ -482,15 +491,15 @@ class MozidraLM:
         H, D, Dv, R = (int(mm[k]) for k in ("heads", "dim", "vdim", "kv_rank"))
         T, dt, dev = h.shape[0], self.dtype, self.device
         qd = self._lin(h, lw.w_in, getattr(lw, "w_in_t", None))                    # [q heads | latent]
-        cache = pages[i]
+        cache, cache_t = pages[i], self.pages_t[i]
         q_rot = torch.empty(T, H, 0, dtype=dt, device=dev)                         # (no rotated part in this family)
         hops.latent_prep(qd, H, D, 0, R, H * D, lw.dkv_norm, self.cfg.norm_eps, inp.positions, None, 0, cache,
-                         inp.slot_mapping, q_rot)
+                         inp.slot_mapping, q_rot, cache_t)
         q_u = qd[:, :H * D].view(T, H, D).transpose(0, 1)                          # [H, T, dim] (strided view)
         q_lat = torch.bmm(q_u, lw.uk_h)                                            # [H, T, R]
         o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
         hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat,
-                         window=lw.window, sink=lw.sink)
+                         cache_t, m.tiles.get(hops.tile_tokens(H)), m.max_keys, window=lw.window, sink=lw.sink)
         ao = torch.bmm(o_lat, lw.uv_ht).transpose(0, 1).reshape(T, H * Dv)         # [T, H vdim]
         return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 

@@ -112,6 +112,11 @@ hipError_t kafka_hy_window_attn(int f32, const void* q, int64_t qs, const void* 
                                 int bt_stride, const int* tok_seg, const int64_t* positions, int H, int G, int D,
                                 int Dv, float scale, int window, const float* sink, void* out, int64_t os, int64_t T,
                                 hipStream_t st);
+int kafka_hy_window_attn_mfma_ok(int page, int D, int Dv, int rep);
+hipError_t kafka_hy_window_attn_mfma(const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
+                                     int bt_stride, const int* items, int n_items, const int64_t* positions, int H,
+                                     int G, int D, int Dv, float scale, int window, const float* sink, void* out,
+                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, hipStream_t st);
 int kafka_hy_grouped_router_max_e();
 int kafka_hy_grouped_router_max_k();
 int kafka_hy_grouped_router_max_g();
@@ -832,6 +837,46 @@ void window_attn(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::
                               out.stride(0), T, stream()));
 }
 
+// the matrix-core kernel: items int32 [n, 4] = (first row, tokens, segment, 0), each at most 32 (token, query head of
+// one key/value head) rows of one segment
+void window_attn_mfma(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor items, int64_t tile_tokens,
+                      at::Tensor positions, int64_t H, int64_t G, double scale, int64_t window, OptT sink,
+                      at::Tensor out, int64_t nsplit, OptT po, OptT pml) {
+  for (const at::Tensor* t : {&q, &kc, &vt, &out})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kBFloat16, "window_attn_mfma: bf16 GPU tensors");
+  rows2d(q, "q"); rows2d(out, "out");
+  const int64_t T = q.size(0);
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && q.size(1) % H == 0 && out.size(0) == T && out.size(1) % H == 0,
+              "window_attn_mfma: heads");
+  const int64_t D = q.size(1) / H, Dv = out.size(1) / H, rep = H / G;
+  paged_kv(kc, vt, G * D, G * Dv, "window_attn_mfma");
+  TORCH_CHECK(kafka_hy_window_attn_mfma_ok(16, (int)D, (int)Dv, (int)rep), "window_attn_mfma: sizes not supported");
+  // 16-byte loads: every query row start must be a multiple of 8 elements
+  TORCH_CHECK(q.stride(0) % 8 == 0 && (reinterpret_cast<uintptr_t>(q.data_ptr()) & 15) == 0,
+              "window_attn_mfma: query alignment");
+  TORCH_CHECK(tile_tokens >= 1 && tile_tokens * rep <= 32, "window_attn_mfma: a tile holds at most 32 rows");
+  TORCH_CHECK(window >= 0, "window_attn_mfma: window");
+  TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.dim() == 2 && bt.stride(1) == 1 && items.is_cuda() &&
+                  items.scalar_type() == at::kInt && items.is_contiguous() && items.dim() == 2 && items.size(1) == 4 &&
+                  positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T, "window_attn_mfma: block tables / items / positions");
+  float *pop = nullptr, *pmlp = nullptr;
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 64, "window_attn_mfma: 1..64 key-range splits");
+  if (nsplit > 1) {
+    TORCH_CHECK(po.has_value() && pml.has_value() && po->is_cuda() && po->scalar_type() == at::kFloat &&
+                    po->is_contiguous() && po->numel() >= nsplit * T * H * Dv && pml->is_cuda() &&
+                    pml->scalar_type() == at::kFloat && pml->is_contiguous() && pml->numel() >= nsplit * T * H * 2,
+                "window_attn_mfma: split workspaces fp32 [splits, T, H Dv] and [splits, T, H, 2]");
+    pop = po->data_ptr<float>(); pmlp = pml->data_ptr<float>();
+  }
+  // the tiles' rows, tokens and segments come from the step plan, which keeps them inside the step
+  HY_HIP(kafka_hy_window_attn_mfma(q.data_ptr(), q.stride(0), kc.data_ptr(), vt.data_ptr(), bt.data_ptr<int>(),
+                                   (int)bt.stride(0), items.data_ptr<int>(), (int)items.size(0),
+                                   positions.data_ptr<int64_t>(), (int)H, (int)G, (int)D, (int)Dv, (float)scale,
+                                   (int)window, sink_ptr(sink, H), out.data_ptr(), out.stride(0), (int)nsplit, pop,
+                                   pmlp, T, stream()));
+}
+
 void moe_topk_grouped(at::Tensor logits, int64_t E, at::Tensor corr, int64_t groups, int64_t keep, double eps,
                       at::Tensor tw, at::Tensor te, OptT gate) {
   rows2d(logits, "logits"); f32t(logits, "logits"); f32t(tw, "weights");
@@ -902,6 +947,12 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_swish_clamp_mul", &swish_clamp_mul);
   m.def("hy_qk_norm_rope_store", &qk_norm_rope_store);
   m.def("hy_window_attn", &window_attn);
+  m.def("hy_window_attn_mfma_ok",
+        [](int page, int D, int Dv, int rep) { return kafka_hy_window_attn_mfma_ok(page, D, Dv, rep) != 0; });
+  m.def("hy_window_attn_mfma", &window_attn_mfma, py::arg("q"), py::arg("kc"), py::arg("vt"), py::arg("bt"),
+        py::arg("items"), py::arg("tile_tokens"), py::arg("positions"), py::arg("H"), py::arg("G"), py::arg("scale"),
+        py::arg("window"), py::arg("sink"), py::arg("out"), py::arg("nsplit") = 1, py::arg("po") = py::none(),
+        py::arg("pml") = py::none());
   m.def("hy_moe_topk_grouped", &moe_topk_grouped);
   m.def("hy_sigmoid_attn_mfma_ok",
         [](int page, int D, int Dv, int rep) { return kafka_hy_sigmoid_attn_mfma_ok(page, D, Dv, rep) != 0; });

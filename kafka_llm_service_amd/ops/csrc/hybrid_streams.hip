@@ -16,6 +16,8 @@
 //                       for the scores (the query row broadcast from LDS), online softmax over 64-key blocks, then
 //                       lane = value channel reading its channel's 16 consecutive tokens of a transposed page; a
 //                       row's keys are visited in order, whatever the batch
+//   window_attn_mfma    the same attention on the matrix cores (bf16): 32 (token, head) rows of one key/value head per
+//                       workgroup, 128-key blocks, online softmax, key-range splits with a merge pass
 //   moe_topk_grouped    softmax over all experts, choice among the best groups by corrected score, normalised weights
 #include "common.h"
 
@@ -34,6 +36,10 @@ __device__ __forceinline__ float ldx(const void* p, bool f32, int64_t i) {
 constexpr int NT = 256;
 constexpr int PAGE = 16;
 constexpr float LOG2E = 1.4426950408889634f;
+
+// Workgroup barrier for LDS hand-overs that leaves global loads (a prefetched next block) in flight: __syncthreads()
+// would drain them as well. This wave's LDS reads and writes are complete (lgkmcnt 0) before it arrives.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // ---- residual streams ----------------------------------------------------------------------------------------------
 constexpr int SMAX = 8;    // streams
@@ -260,6 +266,219 @@ __global__ __launch_bounds__(NT) void window_attn_kernel(const AT* __restrict__ 
   }
 }
 
+// ---- windowed softmax attention on the matrix cores (bf16) --------------------------------------------------------
+// One workgroup (4 waves) per (tile, key/value head): a tile is 32 query rows = (token, query head of this key/value
+// head) pairs of consecutive tokens of one segment (floor(32 / rep) tokens, rep = H / G query heads per key/value
+// head). Keys go by in blocks of 128, from the block that holds the first key the tile's first row sees:
+//   scores   wave w takes keys 32 w .. 32 w + 31 of the block: S = Q K^T as D / 16 MFMA steps (32x32x16), the Q tile
+//            read from LDS, the key rows straight from the paged cache (lane = key, 16 bytes per step), the next
+//            block's rows requested before this block's softmax;
+//   softmax  keys ahead of the row or behind its window count as -inf; row maxima within the wave by lane exchange
+//            and across the four waves through LDS; P = 2^(S - m) goes to LDS as bf16; the row sums stay per lane
+//            and are combined once at the end;
+//   values   wave w owns output columns [32 TW w, 32 TW (w + 1)): O += P V with V read from the page-wise transposed
+//            values (lane = column, 8 consecutive keys = 16 bytes), one page per MFMA step.
+// Scores, maxima, sums and accumulators are fp32. The sink joins the denominator once, at the end. With
+// gridDim.z > 1 the tile's key blocks are dealt to gridDim.z workgroups in contiguous ranges; each leaves its
+// unnormalised accumulators in po [z][T][H Dv] and (row maximum, row sum) in pml [z][T][H][2] for window_merge.
+// Needs 16-token pages, D % 16 == 0, at most 32 query heads per key/value head.
+constexpr int WM_ROWS = 32;
+
+template <int TW, int NKSC>
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(
+    const bf16* __restrict__ q, int64_t qs, const bf16* __restrict__ kc, const bf16* __restrict__ vt,
+    const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
+    int H, int G, int D, int Dv, float scale_log2e, int window, const float* __restrict__ sink,
+    bf16* __restrict__ out, int64_t os, float* __restrict__ po, float* __restrict__ pml, int64_t T) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int nks = D >> 4, qstride = D + 8;
+  bf16* Qs = reinterpret_cast<bf16*>(smem);                       // [32][D + 8]
+  bf16* Ps = Qs + WM_ROWS * qstride;                              // [32][128 + 8]
+  float* mloc = reinterpret_cast<float*>(Ps + WM_ROWS * 136);     // [4][32]
+  int* prow_s = reinterpret_cast<int*>(mloc + 4 * WM_ROWS);       // [32]
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, lr = lane & 31, lh = lane >> 5;
+  const int t0 = items[4 * blockIdx.x], ntok = items[4 * blockIdx.x + 1], sg = items[4 * blockIdx.x + 2];
+  const int g = blockIdx.y, rep = H / G;
+  const int nrows = ntok * rep;
+  for (int i = threadIdx.x; i < WM_ROWS * (D >> 3); i += 256) {
+    const int r = i / (D >> 3), d0 = (i - r * (D >> 3)) << 3;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (r < nrows) v = load_bf16x8(q + (int64_t)(t0 + r / rep) * qs + (int64_t)(g * rep + r % rep) * D + d0);
+    store_bf16x8(Qs + r * qstride + d0, v);
+  }
+  // a row beyond the tile sees no key
+  if (threadIdx.x < WM_ROWS) prow_s[threadIdx.x] = threadIdx.x < nrows ? (int)positions[t0 + threadIdx.x / rep] : -1;
+  const int maxpos = (int)positions[t0 + ntok - 1];
+  __syncthreads();
+  int prow[16];
+  float m[16], lsum[16];
+  f32x16 O[TW];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    prow[i] = prow_s[(i & 3) + 8 * (i >> 2) + 4 * lh];
+    m[i] = -INFINITY;
+    lsum[i] = 0.f;
+  }
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[tw][i] = 0.f;
+  const int* btr = bt + (int64_t)sg * bt_stride;
+  const int Ck = G * D, Cv = G * Dv;
+  const int nblocks = (maxpos >> 7) + 1;
+  const int kbmin = window > 0 ? max(0, (int)positions[t0] - window + 1) >> 7 : 0;
+  const bf16* qrow = Qs + lr * qstride + 8 * lh;
+  bf16x8 kf[NKSC];
+  auto fetch_keys = [&](int kb) {
+    const int kcix = min(kb * 128 + 32 * w + lr, maxpos);  // past the tile's last position: a valid row, masked below
+    const bf16* krow = kc + ((int64_t)btr[kcix >> 4] * PAGE + (kcix & 15)) * Ck + (int64_t)g * D + 8 * lh;
+#pragma unroll
+    for (int ks = 0; ks < NKSC; ++ks)
+      if (ks < nks) kf[ks] = load_bf16x8(krow + 16 * ks);
+  };
+  const int nsplit = gridDim.z;
+  const int bps = (nblocks - kbmin + nsplit - 1) / nsplit;
+  const int kb0 = kbmin + blockIdx.z * bps, kb1 = min(nblocks, kb0 + bps);
+  if (kb0 < kb1 && kb0 * 128 + 32 * w <= maxpos) fetch_keys(kb0);
+  for (int kb = kb0; kb < kb1; ++kb) {
+    const int key = kb * 128 + 32 * w + lr;
+    f32x16 S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+    const bool any = kb * 128 + 32 * w <= maxpos;  // (uniform per wave)
+    if (any) {
+#pragma unroll
+      for (int ks = 0; ks < NKSC; ++ks)
+        if (ks < nks) S = mfma32(load_bf16x8(qrow + 16 * ks), kf[ks], S);
+    }
+    if (kb + 1 < kb1 && (kb + 1) * 128 + 32 * w <= maxpos) fetch_keys(kb + 1);
+    float s[16], mx[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s[i] = (any && key <= prow[i] && (window == 0 || key > prow[i] - window)) ? S[i] * scale_log2e : -INFINITY;
+      float v = s[i];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+      mx[i] = v;
+    }
+    if (lr == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = mx[i];
+    }
+    lds_barrier();
+    float corr[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
+      const float mn = fmaxf(fmaxf(m[i], fmaxf(mloc[r], mloc[32 + r])), fmaxf(mloc[64 + r], mloc[96 + r]));
+      // first block: m = -inf -> corr 0. A range may lie wholly outside a row's window: then mn is still -inf and
+      // the row stays empty (the guards keep inf - inf out)
+      corr[i] = mn == -INFINITY ? 0.f : fast_exp2(m[i] - mn);
+      const float p = mn == -INFINITY ? 0.f : fast_exp2(s[i] - mn);
+      lsum[i] = lsum[i] * corr[i] + p;
+      m[i] = mn;
+      Ps[r * 136 + 32 * w + lr] = (bf16)p;
+    }
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) O[tw][i] *= corr[i];
+    lds_barrier();
+    // ---- values: one page (16 keys) per step
+#pragma unroll
+    for (int k0 = 0; k0 < 8; k0 += 4) {
+      bf16x8 vf[4][TW];  // four pages' value operands in flight together
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if ((kb * 8 + k0 + kk) * 16 > maxpos) break;  // (uniform) pages past the last position
+        const bf16* vp = vt + ((int64_t)btr[kb * 8 + k0 + kk] * Cv + (int64_t)g * Dv) * PAGE + 8 * lh;
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+          const int col = (w * TW + tw) * 32 + lr;
+          bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+          vf[kk][tw] = col < Dv ? load_bf16x8(vp + (int64_t)col * PAGE) : z;
+        }
+      }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if ((kb * 8 + k0 + kk) * 16 > maxpos) break;
+        const bf16x8 a = load_bf16x8(Ps + lr * 136 + 16 * (k0 + kk) + 8 * lh);
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+          if ((w * TW + tw) * 32 < Dv) O[tw] = mfma32(a, vf[kk][tw], O[tw]);
+      }
+    }
+    lds_barrier();
+  }
+  // ---- row sums: across the lanes of a half, then across the waves
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float v = lsum[i];
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    lsum[i] = v;
+  }
+  if (lr == 0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mloc[w * 32 + (i & 3) + 8 * (i >> 2) + 4 * lh] = lsum[i];
+  }
+  lds_barrier();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = (i & 3) + 8 * (i >> 2) + 4 * lh;
+    if (r >= nrows) continue;
+    float l = mloc[r] + mloc[32 + r] + mloc[64 + r] + mloc[96 + r];
+    const int64_t t = t0 + r / rep;
+    const int h = g * rep + r % rep;
+    if (nsplit == 1) {
+      if (sink != nullptr) l += fast_exp2(sink[h] * LOG2E - m[i]);
+      const float inv = 1.0f / l;
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const int col = (w * TW + tw) * 32 + lr;
+        if (col < Dv) out[t * os + (int64_t)h * Dv + col] = (bf16)(O[tw][i] * inv);
+      }
+    } else {
+      const int64_t row = ((int64_t)blockIdx.z * T + t) * H + h;
+      if (w == 0 && lr == 0) {
+        pml[2 * row] = m[i];
+        pml[2 * row + 1] = l;
+      }
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const int col = (w * TW + tw) * 32 + lr;
+        if (col < Dv) po[row * Dv + col] = O[tw][i];
+      }
+    }
+  }
+}
+
+// out[t][h] = sum_z 2^(m_z - m) O_z / (sum_z 2^(m_z - m) l_z + 2^(sink_h - m)) over the key-range splits
+__global__ void window_merge_kernel(const float* __restrict__ po, const float* __restrict__ pml, int nsplit, int64_t T,
+                                    int H, int Dv, const float* __restrict__ sink, bf16* __restrict__ out, int64_t os) {
+  const int64_t th = blockIdx.x;  // t * H + h
+  const int64_t t = th / H;
+  const int h = (int)(th - t * H);
+  const int64_t zs = T * H;
+  float mx = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pml[2 * (z * zs + th)]);
+  float den = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = pml[2 * (z * zs + th)];
+    if (mz != -INFINITY) den += fast_exp2(mz - mx) * pml[2 * (z * zs + th) + 1];
+  }
+  if (sink != nullptr) den += fast_exp2(sink[h] * LOG2E - mx);
+  const float inv = 1.0f / den;
+  for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
+    float a = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float mz = pml[2 * (z * zs + th)];
+      if (mz != -INFINITY) a += fast_exp2(mz - mx) * po[(z * zs + th) * Dv + d];
+    }
+    out[t * os + (int64_t)h * Dv + d] = (bf16)(a * inv);
+  }
+}
+
 // ---- group-limited router ------------------------------------------------------------------------------------------
 constexpr int GR_MAXE = 512;  // experts (8 per lane)
 constexpr int GR_MAXK = 16;
@@ -453,6 +672,35 @@ hipError_t kafka_hy_window_attn(int f32, const void* q, int64_t qs, const void* 
                                                 positions, H, G, D, Dv, scale * LOG2E, window, sink, (AT*)out, os,
                                                 pairs);
   });
+  return hipGetLastError();
+}
+
+// bf16 shapes the matrix-core kernel takes (else the per-wave kernel above runs)
+int kafka_hy_window_attn_mfma_ok(int page, int D, int Dv, int rep) {
+  return page == PAGE && D >= 16 && D % 16 == 0 && D <= 256 && Dv >= 1 && Dv <= 256 && rep >= 1 && rep <= WM_ROWS;
+}
+
+hipError_t kafka_hy_window_attn_mfma(const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
+                                     int bt_stride, const int* items, int n_items, const int64_t* positions, int H,
+                                     int G, int D, int Dv, float scale, int window, const float* sink, void* out,
+                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, hipStream_t st) {
+  if (n_items <= 0) return hipSuccess;
+  if (G < 1 || H % G || window < 0 || !kafka_hy_window_attn_mfma_ok(PAGE, D, Dv, H / G)) return hipErrorInvalidValue;
+  if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (po == nullptr || pml == nullptr))) return hipErrorInvalidValue;
+  const size_t lds = (size_t)WM_ROWS * (D + 8) * 2 + WM_ROWS * 136 * 2 + 5 * WM_ROWS * 4;
+  const dim3 grid((unsigned)n_items, (unsigned)G, (unsigned)nsplit);
+  auto a = [&](auto k) {
+    k<<<grid, 256, lds, st>>>((const bf16*)q, qs, (const bf16*)kc, (const bf16*)vt, bt, bt_stride, items, positions, H,
+                              G, D, Dv, scale * LOG2E, window, sink, (bf16*)out, os, po, pml, T);
+  };
+  const int nks = D / 16, tw = ((Dv + 31) / 32 + 3) / 4;
+  if (tw == 1 && nks <= 4) a(window_attn_mfma_kernel<1, 4>);
+  else if (tw == 1 && nks <= 8) a(window_attn_mfma_kernel<1, 8>);
+  else if (tw == 1) a(window_attn_mfma_kernel<1, 16>);
+  else if (nks <= 8) a(window_attn_mfma_kernel<2, 8>);
+  else a(window_attn_mfma_kernel<2, 16>);
+  if (nsplit > 1)
+    window_merge_kernel<<<(unsigned)(T * H), 64, 0, st>>>(po, pml, nsplit, T, H, Dv, sink, (bf16*)out, os);
   return hipGetLastError();
 }
 

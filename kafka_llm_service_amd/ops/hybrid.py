@@ -1,5 +1,7 @@
-"""Ops of the hybrid decoder family (layer norm, token shift, latent attention, Mamba-2, depth average): GPU tensors
-run the HIP kernels of ``csrc/hybrid.hip``, CPU tensors the fp32 references of ``hybrid_reference.py``.
+"""Ops of the segment-planned decoder families (layer norm, token shift, latent attention, Mamba-2, depth average;
+gated mixers and routed experts; residual streams, windowed attention with sinks, group-limited routing): GPU tensors
+run the HIP kernels of ``csrc/hybrid.hip``, ``hybrid_gated.hip`` and ``hybrid_streams.hip``, CPU tensors the fp32
+references of ``hybrid_reference.py``.
 
 Activations are bf16 or fp32 (the model's dtype, the kernels are built for both); the residual stream, recurrent
 state, norms, softmax and every gate of a recurrence are fp32 in both. A step's rows are described by ``seg`` int32
@@ -503,18 +505,44 @@ def qk_norm_rope_store(qkv, H: int, G: int, D: int, Dv: int, q_w, k_w, eps, posi
                                lam, k_cache, v_cache_t, slot_mapping, q_out)
 
 
+def window_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int) -> bool:
+    """bf16 GPU tensors of sizes the matrix-core kernel takes (16-token pages, key size a multiple of 16, sizes up
+    to 256, at most 32 query heads per key/value head, 16-byte aligned query rows)."""
+    if not (q.is_cuda and q.dtype == torch.bfloat16):
+        return False
+    if q.stride(0) % 8 or q.data_ptr() % 16:  # query rows are read in 16-byte pieces
+        return False
+    return bool(ext().hy_window_attn_mfma_ok(k_cache.shape[1], k_cache.shape[2] // G, v_cache_t.shape[1] // G,
+                                             H // G))
+
+
 def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int, G: int, scale: float, window: int,
-                sink, out) -> None:
+                sink, out, tiles=None, max_keys: int = 0) -> None:
     """Causal softmax attention over paged keys [pages, page, G D] and page-wise transposed values [pages, G Dv, page]:
     row t at position p, head h (key/value head h // (H / G)) sees the keys p - window < j <= p (window 0: all j <= p);
         out = sum_j e^(s_j) v_j / (sum_j e^(s_j) + e^(sink[h])),  s_j = (q . k_j) scale
-    with ``sink`` fp32 [H] (None: no such term). q [T, H D], out [T, H Dv]; scores and weights fp32. One wave per
-    (row, head), keys in order, whatever the batch."""
+    with ``sink`` fp32 [H] (None: no such term). q [T, H D], out [T, H Dv]; scores and weights fp32. With ``tiles``
+    (int32 [n, 4] = (first row, tokens, segment, 0), at most ``sig_tile_tokens(H, G)`` tokens of one segment each) and
+    sizes it takes, bf16 runs on the matrix cores; else one wave per (row, head) on the vector units, keys in order,
+    whatever the batch. ``max_keys`` (the step's longest context) lets a launch of few tiles split its key ranges
+    over more workgroups (``sig_splits``); a merge pass combines them."""
     if window < 0:
         raise ValueError("window_attn: window must be positive (0 = every earlier position)")
     if _gpu(q):
-        ext().hy_window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, int(H), int(G), float(scale),
-                             int(window), sink, out)
+        if tiles is not None and window_attn_mfma_ok(q, k_cache, v_cache_t, H, G):
+            tt = sig_tile_tokens(H, G)
+            if window and max_keys:  # a tile's key range is at most the window and its own tokens long
+                max_keys = min(max_keys, window + tt)
+            ns = sig_splits(tiles.shape[0] * G, max_keys) if max_keys else 1
+            po = pml = None
+            if ns > 1:
+                po = torch.empty(ns, q.shape[0], out.shape[1], dtype=torch.float32, device=q.device)
+                pml = torch.empty(ns, q.shape[0], H, 2, dtype=torch.float32, device=q.device)
+            ext().hy_window_attn_mfma(q, k_cache, v_cache_t, block_tables, tiles, tt, positions, int(H), int(G),
+                                      float(scale), int(window), sink, out, ns, po, pml)
+        else:
+            ext().hy_window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, int(H), int(G), float(scale),
+                                 int(window), sink, out)
     else:
         ref.window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out)
 

@@ -241,9 +241,10 @@ class MozidraLM:
         return sum(w.numel() * w.element_size() for w in ws if self._streamable(w))
 
     def enable_stream_weights(self, tiled_only: bool = False) -> int:
-        """Wave-tiled copies of the bias-free projections (ops.tile_weight) so that decode-sized steps (<=
-        ops.STREAM_MAX_M rows) run them on the framework's weight-streaming MFMA GEMM; prefill-sized steps and shapes
-        the kernel does not take stay on hipBLASLt. bf16 only. Returns the added bytes."""
+        """Wave-tiled copies of the projections (ops.tile_weight) and of the experts (ops.tile_experts) so that
+        decode-sized steps (<= ops.STREAM_MAX_M rows; experts: <= hops.MOE_STREAM_MAX_T) run them on the framework's
+        weight-streaming MFMA kernels; prefill-sized steps and shapes the kernels do not take stay on hipBLASLt and
+        the expert-sorted GEMMs. bf16 only. Returns the added bytes."""
         added = 0
         for lw in self.layers:
             for n in self.STREAMED:
@@ -251,6 +252,14 @@ class MozidraLM:
                 if self._streamable(w):
                     setattr(lw, n + "_t", ops.tile_weight(w))
                     added += w.numel() * w.element_size()
+            if lw.z is not None and lw.w_gu.is_cuda and lw.w_gu.dtype == torch.bfloat16 and \
+                    hops.moe_grouped_ok(torch.empty(1, lw.w_gu.shape[2], dtype=lw.w_gu.dtype, device=self.device),
+                                        lw.w_gu, lw.w_down) and \
+                    ops.stream_moe_supported(lw.w_gu.shape[1], lw.w_gu.shape[2]) and \
+                    ops.stream_moe_supported(lw.w_down.shape[1], lw.w_down.shape[2]):
+                lw.w_gu_t = ops.tile_experts(lw.w_gu, glu=True)   # expert feed-forwards: grouped streaming kernel
+                lw.w_down_t = ops.tile_experts(lw.w_down)
+                added += (lw.w_gu.numel() + lw.w_down.numel()) * lw.w_gu.element_size()
         if self._streamable(self.head):
             self.head_t = ops.tile_weight(self.head)
             added += self.head.numel() * self.head.element_size()
@@ -510,7 +519,8 @@ class MozidraLM:
         tw, te, gate = hops.moe_router_grouped(h, lw.router, lw.correction, z["top"], z["groups"], z["keep"],
                                                ROUTE_EPS, extra_gate=lw.sh_gu is not None)
         out = torch.empty(T, d, dtype=torch.float32, device=dev)
-        hops.moe_experts(h, lw.w_gu, lw.w_down, tw, te, out, act="swish_clamp", limit=z["limit"], alpha=SWISH_ALPHA)
+        hops.moe_experts(h, lw.w_gu, lw.w_down, tw, te, out, getattr(lw, "w_gu_t", None), getattr(lw, "w_down_t", None),
+                         act="swish_clamp", limit=z["limit"], alpha=SWISH_ALPHA)
         ys = None
         if lw.sh_gu is not None:
             a = torch.empty(T, z["shared_ff"], dtype=dt, device=dev)

@@ -512,19 +512,25 @@ def stream_moe_supported(N: int, K: int) -> bool:
 GROUPED_PIN = True
 
 
-def grouped_stream_glu(x: torch.Tensor, wt: torch.Tensor, r: "MoERouting", e_lo: int = 0) -> torch.Tensor:
+def grouped_stream_glu(x: torch.Tensor, wt: torch.Tensor, r: "MoERouting", e_lo: int = 0, limit: float = 0.0,
+                       alpha: float = 1.0) -> torch.Tensor:
     """silu(gate) * up for every routed (token, local expert) entry, rows in expert-sorted order [n_ent, F]: the
-    weight-streaming grouped kernel on GLU-tiled expert weights (``tile_experts(w13, glu=True)``)."""
+    weight-streaming grouped kernel on GLU-tiled expert weights (``tile_experts(w13, glu=True)``). With ``limit`` > 0
+    the clamped form g' sigmoid(alpha g') (u' + 1), g' = min(gate, limit), u' = clamp(up, -limit, limit)."""
     T = x.shape[0]
     n_ent = r.perm_tok.numel()
     F = wt.shape[1] * 16
     y = torch.empty(n_ent, F, dtype=x.dtype, device=x.device)
     if _gpu(x):
         ext().wstream_grouped(x, wt, r.perm_tok, r.perm_w, r.expert_off, int(e_lo), int(T), True, y, None,
-                              GROUPED_PIN)
+                              GROUPED_PIN, float(limit), float(alpha))
         return y
     h = ref_grouped(x, untile_experts(wt, glu=True), r, e_lo, gather=True)
-    y.copy_(ref.silu_mul(h))
+    if limit > 0:
+        g, u = h[:, :F].float().clamp(max=limit), h[:, F:].float().clamp(min=-limit, max=limit)
+        y.copy_((g * torch.sigmoid(alpha * g) * (u + 1.0)).to(y.dtype))
+    else:
+        y.copy_(ref.silu_mul(h))
     return y
 
 

@@ -8,7 +8,8 @@
 //   stream_step         one pass over S residual streams [S][T][d] (fp32): the write of a sublayer's output (all
 //                       streams at once from the old ones: x_r <- sum_s M[s][r] x_s + b_r y), the next sublayer's read
 //                       u = sum_s a_s x_s with its RMS norm, and the plain sum - every part optional. One workgroup
-//                       per row; a row's read values stay in registers between the statistics and the scaling.
+//                       per row; a row's columns are loaded in one round, and its read values stay in registers
+//                       between the statistics and the scaling.
 //   swish_clamp_mul     g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
 //   qk_norm_rope_store  RMS norm over the whole q and the whole k projection, rotation of dimension pairs (2i, 2i + 1),
 //                       value mix with an earlier layer's values, paged key / transposed value store
@@ -42,9 +43,11 @@ constexpr float LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // ---- residual streams ----------------------------------------------------------------------------------------------
-constexpr int SMAX = 8;    // streams
-constexpr int UREG = 16;   // read values a thread keeps between the two passes (rows up to NT * UREG wide; wider rows
-                           // recompute them from the streams just written)
+constexpr int SMAX = 16;   // streams
+// columns of a row a thread keeps in registers (all S streams of each): rows up to NT * stream_nv(S) wide are loaded in
+// one round of independent loads, written once, and their read values wait in registers for the row's mean square;
+// wider rows walk the rest column by column and recompute the read values from the streams just written
+__host__ __device__ constexpr int stream_nv(int S) { return S <= 4 ? 16 : S <= 8 ? 8 : 4; }
 
 template <int S>
 __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs, int64_t s_stride, int64_t t_stride,
@@ -55,10 +58,12 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
                                                          const float* __restrict__ rd, const float* __restrict__ nw,
                                                          float eps, void* __restrict__ out, int64_t os, bool out_f32,
                                                          float* __restrict__ total, int64_t ts, int d) {
+  constexpr int NV = stream_nv(S);
   __shared__ float red[NT / 64];
   __shared__ float cM[SMAX * SMAX], cb[SMAX], ca[SMAX];
   const int64_t t = blockIdx.x;
-  if (threadIdx.x < S * S && mix != nullptr) cM[threadIdx.x] = mix[threadIdx.x];
+  for (int i = threadIdx.x; i < S * S; i += NT)
+    if (mix != nullptr) cM[i] = mix[i];
   if (threadIdx.x < S) {
     if (wr != nullptr) cb[threadIdx.x] = wr[threadIdx.x];
     if (rd != nullptr) ca[threadIdx.x] = rd[threadIdx.x];
@@ -66,29 +71,73 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
   __syncthreads();
   float* xr = xs + t * t_stride;
   const float rs2 = y2 != nullptr ? row_scale[t] : 0.f;
-  float ureg[UREG];
+  // new stream values of one column from the old ones and the sublayer's output
+  auto write = [&](float (&x)[S], float yv) {
+    float nx[S];
+#pragma unroll
+    for (int r = 0; r < S; ++r) {
+      float v = cb[r] * yv;
+#pragma unroll
+      for (int s = 0; s < S; ++s) v += cM[s * S + r] * x[s];
+      nx[r] = v;
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s) x[s] = nx[s];
+  };
+  auto read = [&](const float (&x)[S]) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < S; ++s) u += ca[s] * x[s];
+    return u;
+  };
+  float xv[NV][S], yv[NV];
   float acc = 0.f;
-  int it = 0;
-  for (int i = threadIdx.x; i < d; i += NT, ++it) {
+  // the register part: every load of the row's first NT * NV columns is issued before anything is stored
+#pragma unroll
+  for (int it = 0; it < NV; ++it) {
+    const int i = threadIdx.x + it * NT;
+    yv[it] = 0.f;
+    if (i < d) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) xv[it][s] = xr[s * s_stride + i];
+      if (mix != nullptr) {
+        yv[it] = ldx(y, y_f32, t * ys + i);
+        if (y2 != nullptr) yv[it] += rs2 * ldx(y2, y2_f32, t * y2s + i);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NV; ++it) {
+    const int i = threadIdx.x + it * NT;
+    if (i < d) {
+      if (mix != nullptr) {
+        write(xv[it], yv[it]);
+#pragma unroll
+        for (int s = 0; s < S; ++s) xr[s * s_stride + i] = xv[it][s];
+      }
+      if (total != nullptr) {
+        float v = 0.f;
+#pragma unroll
+        for (int s = 0; s < S; ++s) v += xv[it][s];
+        total[t * ts + i] = v;
+      }
+      if (rd != nullptr) {
+        const float u = read(xv[it]);
+        acc += u * u;
+        yv[it] = u;  // (the sublayer output is used up: its register keeps the read value)
+      }
+    }
+  }
+  for (int i = threadIdx.x + NV * NT; i < d; i += NT) {
     float x[S];
 #pragma unroll
     for (int s = 0; s < S; ++s) x[s] = xr[s * s_stride + i];
     if (mix != nullptr) {
-      float yv = ldx(y, y_f32, t * ys + i);
-      if (y2 != nullptr) yv += rs2 * ldx(y2, y2_f32, t * y2s + i);
-      float nx[S];
+      float v = ldx(y, y_f32, t * ys + i);
+      if (y2 != nullptr) v += rs2 * ldx(y2, y2_f32, t * y2s + i);
+      write(x, v);
 #pragma unroll
-      for (int r = 0; r < S; ++r) {
-        float v = cb[r] * yv;
-#pragma unroll
-        for (int s = 0; s < S; ++s) v += cM[s * S + r] * x[s];
-        nx[r] = v;
-      }
-#pragma unroll
-      for (int s = 0; s < S; ++s) {
-        x[s] = nx[s];
-        xr[s * s_stride + i] = nx[s];
-      }
+      for (int s = 0; s < S; ++s) xr[s * s_stride + i] = x[s];
     }
     if (total != nullptr) {
       float v = 0.f;
@@ -97,28 +146,27 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
       total[t * ts + i] = v;
     }
     if (rd != nullptr) {
-      float u = 0.f;
-#pragma unroll
-      for (int s = 0; s < S; ++s) u += ca[s] * x[s];
+      const float u = read(x);
       acc += u * u;
-      if (it < UREG) ureg[it] = u;
     }
   }
   if (rd == nullptr) return;
   const float rs = 1.0f / sqrtf(block_sum<NT>(acc, red) / (float)d + eps);
-  it = 0;
-  for (int i = threadIdx.x; i < d; i += NT, ++it) {
-    float u;
-    if (it < UREG) {
-      u = ureg[it];
-    } else {  // (this thread's own writes of the first pass)
-      u = 0.f;
-#pragma unroll
-      for (int s = 0; s < S; ++s) u += ca[s] * xr[s * s_stride + i];
-    }
+  auto store = [&](int i, float u) {
     const float v = u * rs * nw[i];
     if (out_f32) reinterpret_cast<float*>(out)[t * os + i] = v;
     else reinterpret_cast<bf16*>(out)[t * os + i] = (bf16)v;
+  };
+#pragma unroll
+  for (int it = 0; it < NV; ++it) {
+    const int i = threadIdx.x + it * NT;
+    if (i < d) store(i, yv[it]);
+  }
+  for (int i = threadIdx.x + NV * NT; i < d; i += NT) {  // (this thread's own writes of the first pass)
+    float x[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) x[s] = xr[s * s_stride + i];
+    store(i, read(x));
   }
 }
 
@@ -627,7 +675,15 @@ hipError_t kafka_hy_stream_step(float* xs, int64_t s_stride, int64_t t_stride, i
     case 5: a(stream_step_kernel<5>); break;
     case 6: a(stream_step_kernel<6>); break;
     case 7: a(stream_step_kernel<7>); break;
-    default: a(stream_step_kernel<8>); break;
+    case 8: a(stream_step_kernel<8>); break;
+    case 9: a(stream_step_kernel<9>); break;
+    case 10: a(stream_step_kernel<10>); break;
+    case 11: a(stream_step_kernel<11>); break;
+    case 12: a(stream_step_kernel<12>); break;
+    case 13: a(stream_step_kernel<13>); break;
+    case 14: a(stream_step_kernel<14>); break;
+    case 15: a(stream_step_kernel<15>); break;
+    default: a(stream_step_kernel<16>); break;
   }
   return hipGetLastError();
 }

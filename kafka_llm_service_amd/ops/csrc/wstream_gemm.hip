@@ -661,7 +661,8 @@ __global__ __launch_bounds__(256 * KW) void wstream_gemm_kernel(const bf16* __re
 // [expert_off[e], expert_off[e + 1]) read on the device (no host sync after the router); workgroups past the end
 // of their expert's segment exit at once, and row tiles past it skip their MFMAs (wave-uniform).
 //   GATHER: A row = X[perm_tok[entry]] (token activations), else X[entry] (expert-sorted intermediate).
-//   Epilogue GLU (GLU-interleaved tiles): Y[entry, :N/2] = silu(gate) * up, bf16 — the SwiGLU of the expert MLP.
+//   Epilogue GLU (GLU-interleaved tiles): Y[entry, :N/2] = silu(gate) * up, bf16 — the SwiGLU of the expert MLP; with
+//   glu_limit > 0 the clamped form g' sigmoid(glu_alpha g') (u' + 1), g' = min(gate, limit), u' = clamp(up, +-limit).
 //   Epilogue COMBINE: out_f32[perm_tok[entry], n] += perm_w[entry] * y (a token gets exactly k contributions).
 // (MT = 4: at most 256 registers so two workgroups share a CU — left free the compiler took 316, one wave per SIMD:
 // the 128-row expert tiles streamed 8 % slower, Mixtral 128 threads 5,155 vs 5,234 tok/s, profiles/r06/mixtral/;
@@ -673,7 +674,8 @@ __global__ __launch_bounds__(256, MT == 4 ? 2 : 1) void wstream_grouped_kernel(c
                                                                const float* __restrict__ perm_w,
                                                                const int* __restrict__ expert_off, int e_lo,
                                                                bf16* __restrict__ Y, int64_t ldy,
-                                                               float* __restrict__ out, int64_t ldo) {
+                                                               float* __restrict__ out, int64_t ldo, float glu_limit,
+                                                               float glu_alpha) {
   constexpr int ROWS = 32 * MT;
   constexpr int CPR = KC / 8;
   constexpr int XL = ROWS * CPR / 256;
@@ -792,8 +794,14 @@ __global__ __launch_bounds__(256, MT == 4 ? 2 : 1) void wstream_grouped_kernel(c
       for (int i = 0; i < 16; ++i) {
         const int m = mt * 32 + (i & 3) + 8 * (i >> 2) + 4 * h;
         if (m < rows) {
-          const float g = acc[mt][i], u = red[(((w >> 1) * MT + mt) * 16 + i) * 64 + lane];
-          Y[(int64_t)(seg0 + row0 + m) * ldy + n] = (bf16)(g / (1.0f + __expf(-g)) * u);
+          float g = acc[mt][i], u = red[(((w >> 1) * MT + mt) * 16 + i) * 64 + lane];
+          float a = 1.0f;
+          if (glu_limit > 0.f) {  // (uniform) the clamped form
+            g = fminf(g, glu_limit);
+            u = fminf(fmaxf(u, -glu_limit), glu_limit) + 1.0f;
+            a = glu_alpha;
+          }
+          Y[(int64_t)(seg0 + row0 + m) * ldy + n] = (bf16)(g / (1.0f + __expf(-a * g)) * u);
         }
       }
   } else {
@@ -1001,7 +1009,7 @@ extern "C" hipError_t kafka_launch_wstream_grouped(const bf16* X, int64_t ldx, c
                                                   int K, const int* perm_tok, const float* perm_w,
                                                   const int* expert_off, int e_lo, int max_rows, int gather,
                                                   bf16* Y, int64_t ldy, float* out, int64_t ldo, int pin,
-                                                  hipStream_t st) {
+                                                  float glu_limit, float glu_alpha, hipStream_t st) {
   if (max_rows < 1 || e_local < 1) return hipSuccess;
   if (N % 64 != 0 || K % 256 != 0 || (out == nullptr) == (Y == nullptr)) return hipErrorInvalidValue;
   // MT = 4 (128-row tiles on 128-deep K chunks) for large steps: with 64-row tiles every
@@ -1023,10 +1031,12 @@ extern "C" hipError_t kafka_launch_wstream_grouped(const bf16* X, int64_t ldx, c
     constexpr int KC_ = MT_ == 4 ? 128 : 256;                                                                  \
     if (pin)                                                                                                   \
       wstream_grouped_kernel<MT_, KC_, G_, C_, true><<<grid, 256, 0, st>>>(X, ldx, wt, N, K, perm_tok, perm_w,      \
-                                                                           expert_off, e_lo, Y, ldy, out, ldo);  \
+                                                                           expert_off, e_lo, Y, ldy, out, ldo,   \
+                                                                           glu_limit, glu_alpha);               \
     else                                                                                                       \
       wstream_grouped_kernel<MT_, KC_, G_, C_, false><<<grid, 256, 0, st>>>(X, ldx, wt, N, K, perm_tok, perm_w,     \
-                                                                            expert_off, e_lo, Y, ldy, out, ldo); \
+                                                                            expert_off, e_lo, Y, ldy, out, ldo,  \
+                                                                            glu_limit, glu_alpha);              \
   } while (0)
   const bool comb = out != nullptr;
   if (MT == 1) {

@@ -412,15 +412,16 @@ def moe_experts(h, w_gu, w_down, topk_w, topk_e, out, w_gu_t=None, w_down_t=None
     gathered rows, silu * up, down GEMM with the weighted combine in its epilogue (fp32 adds, two entries per row
     commute), or the grouped weight-streaming kernels when tiled expert weights are given and the step is small -
     everything else is evaluated per (row, expert) pair by ``moe_rows``. ``act`` as in ``moe_rows`` (the streaming
-    kernels have silu built in; another activation runs between the two expert-sorted GEMMs)."""
+    kernel applies it in its epilogue; between the two expert-sorted GEMMs it is a launch of its own)."""
     from kafka_llm_service_amd import ops
 
     T = h.shape[0]
     if T and moe_grouped_ok(h, w_gu, w_down):
         r = ops.moe_sort(topk_w, topk_e, w_gu.shape[0])
         out.zero_()
-        if act == "silu" and w_gu_t is not None and w_down_t is not None and T <= MOE_STREAM_MAX_T:
-            a = ops.grouped_stream_glu(h, w_gu_t, r)
+        if w_gu_t is not None and w_down_t is not None and T <= MOE_STREAM_MAX_T:
+            lim, al = _glu_act(act, limit, alpha)
+            a = ops.grouped_stream_glu(h, w_gu_t, r, limit=lim, alpha=al)
             ops.grouped_stream_combine(a, w_down_t, r, T, out)
         else:
             gu = ops.grouped_gemm(h, w_gu, r, gather=True)
@@ -446,7 +447,7 @@ def add2(x, y1, y2=None, norm_w=None, eps=0.0, out=None) -> None:
 
 
 # ---- hyper-connected residual streams, windowed softmax attention with sinks, group-limited routing -----------------
-STREAM_MAX = 8   # residual streams the stream kernel keeps in registers
+STREAM_MAX = 16   # residual streams the stream kernel takes
 
 
 def stream_step(xs, y=None, mix=None, write=None, read=None, norm_w=None, eps=0.0, out=None, y2=None,

@@ -152,7 +152,7 @@ def bench_sharp():
 
 # ---- mechanisms alone ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("S,d", [(3, 70), (1, 33), (4, 4500), (8, 130)])
+@pytest.mark.parametrize("S,d", [(3, 70), (1, 33), (4, 4500), (8, 2300), (13, 1100)])
 def test_stream_step(device, S, d):
     """Write, read + norm and sum of the streams, each alone and together, against the plain stream step; rows wider
     than the kernel keeps in registers; bf16 and fp32 sublayer outputs; a second output with a row gate."""
@@ -579,6 +579,31 @@ def test_clamped_experts_on_the_matrix_cores():
     assert (out.cpu() - ref).abs().max() < 0.03 * ref.abs().max()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [1, 70, 300])
+def test_clamped_experts_on_the_streaming_kernel(T):
+    """Tiled expert weights: steps of few rows run the grouped weight-streaming kernel with the clamped activation in
+    its epilogue."""
+    from kafka_llm_service_amd import ops
+
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(T)
+    E, k, d, ff, limit = 8, 2, 256, 256, 0.6
+    h = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    w_gu = (torch.randn(E, 2 * ff, d, generator=g) / 8).to(torch.bfloat16)
+    w_dn = (torch.randn(E, d, ff, generator=g) / 8).to(torch.bfloat16)
+    te = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    tw = torch.rand(T, k, generator=g)
+    assert ops.stream_moe_supported(2 * ff, d) and ops.stream_moe_supported(d, ff)
+    gu_t, dn_t = ops.tile_experts(w_gu.to(dev), glu=True), ops.tile_experts(w_dn.to(dev))
+    out = torch.empty(T, d, device=dev)
+    hops.moe_experts(h.to(dev), w_gu.to(dev), w_dn.to(dev), tw.to(dev), te.to(dev), out, gu_t, dn_t, act="swish_clamp",
+                     limit=limit, alpha=mz.SWISH_ALPHA)
+    ref = torch.empty(T, d)
+    hops.moe_experts(h, w_gu, w_dn, tw, te, ref, act="swish_clamp", limit=limit, alpha=mz.SWISH_ALPHA)
+    assert (out.cpu() - ref).abs().max() < 0.03 * ref.abs().max()
+
+
 # ---- the model in the engine ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -697,6 +722,7 @@ def test_preset_sizes_matrix_cores_and_streamed_projections():
     eng = b.engine("cuda:0", "bfloat16")
     eng.model.enable_stream_weights()
     assert eng.model.stream and eng.model.attn_tile_tokens and eng.model.pages_t[0] is not None
+    assert hasattr(eng.model.layers[0], "w_gu_t")
     whole = feed_all(eng, "w", t, [200])
     assert mean_err(whole, b.oracle(t)) < 0.05
     for cuts in ([150, 1], [3, 64, 5]):

@@ -270,8 +270,9 @@ def test_windowed_attention_single_keys(device, H, G, D, Dv, window, rot):
     q, k, v, vf = seqs[0]
     qh, kh = q.view(n0, H, D), k.view(n0, G, D)
     w = window or 10 ** 6
+    # (row 97 is fed alone, as a decoded token: its window's last visible key and the one just outside it)
     spots = [(149, 0), (149, 149), (140, 127), (140, 128), (100, 15), (100, 16), (120, max(0, 120 - w + 1)),
-             (121, max(0, 121 - w)), (149, 3)]
+             (121, max(0, 121 - w)), (149, 3), (97, max(0, 97 - w + 1)), (97, max(0, 97 - w))]
     for i, (at, key) in enumerate(spots):
         h = i % H
         kh[key, h // (H // G)] = torch.randn(D, generator=g) * 3.0
@@ -326,7 +327,7 @@ def test_windowed_attention_matrix_cores(H, G, D, Dv, window, n):
     k = torch.randn(n, G, D, generator=g)
     v = torch.randn(n, G, Dv, generator=g)
     spots = [(n - 1, 0), (n - 1, n - 1), (140, 127), (140, 128), (100, 15), (120, max(0, 120 - w + 1)),
-             (121, max(0, 121 - w)), (n - 1, max(0, n - w)), (n - 2, max(0, n - 2 - w))]
+             (121, max(0, 121 - w)), (n - 1, max(0, n - w)), (n - 2, max(0, n - 2 - w)), (n - 1, max(0, n - 1 - w))]
     for i, (at, key) in enumerate(spots):
         h = i % H
         k[key, h // (H // G)] = torch.randn(D, generator=g) * 2.0
@@ -413,8 +414,9 @@ def test_latent_attention_window_and_sink(device, H, R, window):
     g = torch.Generator().manual_seed(H + R)
     n = 150
     w = window or 10 ** 6
+    # (row 97 is fed alone, as a decoded token: its window's last visible key and the one just outside it)
     spots = [(149, 0), (149, 149), (140, 127), (140, 128), (100, 15), (100, 16), (120, max(0, 120 - w + 1)),
-             (121, max(0, 121 - w))]
+             (121, max(0, 121 - w)), (97, max(0, 97 - w + 1)), (97, max(0, 97 - w))]
     c, ql, sink, want = _latent_case(g, n, H, R, window, spots)
     pg = Paged(device, [n], seed=R)
     cache = torch.zeros(pg.n_pages, 16, R, device=device)
@@ -448,7 +450,7 @@ def test_latent_attention_matrix_cores_window_and_sink(H, R, window, n):
     g = torch.Generator().manual_seed(H * R)
     w = window or 10 ** 6
     spots = [(n - 1, 0), (n - 1, n - 1), (140, 127), (140, 128), (100, 15), (120, max(0, 120 - w + 1)),
-             (121, max(0, 121 - w)), (n - 1, max(0, n - w)), (n - 2, max(0, n - 2 - w))]
+             (121, max(0, 121 - w)), (n - 1, max(0, n - w)), (n - 2, max(0, n - 2 - w)), (n - 1, max(0, n - 1 - w))]
     c, ql, sink, _ = _latent_case(g, n, H, R, window, spots)
     c = c / c.pow(2).mean(-1, keepdim=True).sqrt()
     cb, qb = c.to(torch.bfloat16), ql.to(torch.bfloat16)

@@ -72,7 +72,7 @@ class EngineConfig:
     dp_attention: bool = False
     eos_token_ids: list[int] = field(default_factory=list)
     # activation / weight dtype: "bfloat16", or "float32" (every matrix product and activation in true fp32) for the
-    # model families whose kernels are built for it (Budurax)
+    # model families whose kernels are built for it (models.config.FP32_ARCHS)
     dtype: str = "bfloat16"
 
     def resolve_device(self) -> torch.device:

@@ -509,7 +509,8 @@ class MozidraLM:
         o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
         hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat,
                          cache_t, m.tiles.get(hops.tile_tokens(H)), m.max_keys, window=lw.window, sink=lw.sink)
-        ao = torch.bmm(o_lat, lw.uv_ht).transpose(0, 1).reshape(T, H * Dv)         # [T, H vdim]
+        ao = torch.empty(T, H * Dv, dtype=dt, device=dev)
+        torch.bmm(o_lat, lw.uv_ht, out=ao.view(T, H, Dv).transpose(0, 1))          # head h -> columns [h vdim, (h + 1) vdim)
         return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 
     def _experts(self, lw, h):

@@ -5,7 +5,7 @@ Residual streams. Instead of one residual x the model carries ``streams`` copies
 embedding at the start). A sublayer (mixer or feed-forward) with coefficients a (read, [S]), M (mix, [S, S], indexed
 [from, to]) and b (write, [S]) does
 
-    u = sum_s a_s x_s        y = sublayer(rms_norm(u) * (1 + w))        x_r <- sum_s M[s, r] x_s + b_r y   (all r at once)
+    u = sum_s a_s x_s      y = sublayer(rms_norm(u) * (1 + w))      x_r <- sum_s M[s, r] x_s + b_r y   (all r at once)
 
 and the model's output reads the sum of the streams through the final norm (weights stored around zero: 1 + w). A
 config without ``streams`` is the plain pre-norm residual, which is the same computation with S = 1 and a = M = b = 1.
@@ -425,7 +425,7 @@ class MozidraLM:
         patterns for the debug checks."""
         dev, dt = self.device, self.dtype
         pages = []
-        self.pages_t = []  # page-wise transposed latent copies [blocks, kv_rank, 16] where the matrix-core kernel applies
+        self.pages_t = []  # page-wise transposed latent copies [blocks, kv_rank, 16] for the matrix-core kernel
         for lw in self.layers:
             m = lw.m
             if lw.type == "attention":
@@ -467,7 +467,8 @@ class MozidraLM:
             else:
                 ye, ys, gate, last = y, None, None, lw.hc1
             if nxt is not None:
-                hops.stream_step(xs, ye, last.M, last.b, nxt.hc1.a, nxt.norm1, eps, h, y2=ys, row_scale=gate, total=total)
+                hops.stream_step(xs, ye, last.M, last.b, nxt.hc1.a, nxt.norm1, eps, h, y2=ys, row_scale=gate,
+                                 total=total)
             else:
                 hops.stream_step(xs, ye, last.M, last.b, y2=ys, row_scale=gate, total=total)
             if layers_out is not None:
@@ -481,7 +482,7 @@ class MozidraLM:
         mm = lw.m
         H, G, D, Dv = (int(mm[k]) for k in ("heads", "kv_heads", "dim", "vdim"))
         T, dt, dev = h.shape[0], self.dtype, self.device
-        qkv = self._lin(h, lw.w_in, getattr(lw, "w_in_t", None), lw.b_in)                                # [q | k | v], biases added
+        qkv = self._lin(h, lw.w_in, getattr(lw, "w_in_t", None), lw.b_in)   # [q | k | v], biases added
         k_cache, v_cache_t = pages[i]
         q = torch.empty(T, H * D, dtype=dt, device=dev)
         vf = step.get(lw.vmix_from) if lw.vmix_from is not None else None          # (rows, first value column)
@@ -510,7 +511,7 @@ class MozidraLM:
         hops.latent_attn(q_lat, q_rot, cache, m.block_tables, m.tok_seg, m.seg, inp.positions, lw.scale, o_lat,
                          cache_t, m.tiles.get(hops.tile_tokens(H)), m.max_keys, window=lw.window, sink=lw.sink)
         ao = torch.empty(T, H * Dv, dtype=dt, device=dev)
-        torch.bmm(o_lat, lw.uv_ht, out=ao.view(T, H, Dv).transpose(0, 1))          # head h -> columns [h vdim, (h + 1) vdim)
+        torch.bmm(o_lat, lw.uv_ht, out=ao.view(T, H, Dv).transpose(0, 1))          # head h -> its vdim columns
         return self._lin(ao, lw.o, getattr(lw, "o_t", None))
 
     def _experts(self, lw, h):

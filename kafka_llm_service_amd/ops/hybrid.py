@@ -488,7 +488,7 @@ def swish_clamp_mul(gu, limit: float, alpha: float, out) -> None:
 def qk_norm_rope_store(qkv, H: int, G: int, D: int, Dv: int, q_w, k_w, eps, positions, cos_sin, rot_dims: int,
                        v_first, v_first_off: int, lam: float, k_cache, v_cache_t, slot_mapping, q_out) -> None:
     """Attention inputs from the fused projection row [q (H D) | k (G D) | v (G Dv)]:
-      * RMS norm over the WHOLE q part and over the whole k part (weights fp32 [H D], [G D]), before the split into heads;
+      * RMS norm over the WHOLE q part and over the whole k part (weights fp32 [H D], [G D]), before the head split;
       * rotation of the dimension pairs (2i, 2i + 1), i < rot_dims / 2, of every q and k head by the row's position
         (``cos_sin`` fp32 [positions, rot_dims] = cos | sin per frequency; rot_dims = 0 and no table: no rotation);
       * values: with ``v_first`` (rows [T, ...] whose value columns start at ``v_first_off``) v <- (1 - lam) v + lam

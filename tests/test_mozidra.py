@@ -59,14 +59,17 @@ def cfg_a(scale=None):
 
 
 def cfg_b():
-    """Ones and equal values: no streams, one head, as many key/value heads as query heads, one expert of one, one group,
-    no shared expert, a window of one token (a row sees itself only), a full rotation, key and value sizes equal."""
+    """Ones and equal values: no streams, one head, as many key/value heads as query heads, one expert of one, one
+    group, no shared expert, a window of one token (a row sees itself only), a full rotation, key and value sizes
+    equal."""
     return {"architecture": "Mozidra", "vocab": 97, "width": 48, "norm": {"eps": 1e-6},
             "layers": [{"type": "attention", "mixer": _attn(1, 1, 16, 16, window=1, rot=16, v_mix=True),
                         "mlp": _moe(1, 1, 40, None, 0)},
-                       {"type": "latent_attention", "mixer": _lat(1, 16, 16, 16, window=1000), "mlp": _moe(2, 2, 8, (1, 1), 8)},
+                       {"type": "latent_attention", "mixer": _lat(1, 16, 16, 16, window=1000),
+                        "mlp": _moe(2, 2, 8, (1, 1), 8)},
                        {"type": "attention", "mixer": _attn(3, 1, 8, 16, window=2, rot=2, v_mix=True), "mlp": None},
-                       {"type": "latent_attention", "mixer": _lat(2, 8, 8, 8, window=0), "mlp": _moe(4, 1, 8, (2, 2), 8)}]}
+                       {"type": "latent_attention", "mixer": _lat(2, 8, 8, 8, window=0),
+                        "mlp": _moe(4, 1, 8, (2, 2), 8)}]}
 
 
 def cfg_s1():
@@ -314,7 +317,8 @@ def test_windowed_attention_single_keys(device, H, G, D, Dv, window, rot):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,D,Dv,window,n", [(8, 2, 32, 48, 40, 300), (4, 4, 16, 20, 129, 700), (32, 1, 64, 96, 0, 200),
+@pytest.mark.parametrize("H,G,D,Dv,window,n", [(8, 2, 32, 48, 40, 300), (4, 4, 16, 20, 129, 700),
+                                               (32, 1, 64, 96, 0, 200),
                                                (6, 3, 96, 96, 1, 150), (8, 2, 128, 256, 1000, 1500),
                                                (8, 1, 64, 80, 150, 520)])
 def test_windowed_attention_matrix_cores(H, G, D, Dv, window, n):
@@ -375,7 +379,8 @@ def test_attention_without_sink_mix_and_rotation(device):
     """The optional parts switched off: no sink, no earlier values, no rotation, no window."""
     g = torch.Generator().manual_seed(2)
     n, H, G, D, Dv = 40, 4, 2, 12, 9
-    q, k, v = torch.randn(n, H * D, generator=g), torch.randn(n, G * D, generator=g), torch.randn(n, G * Dv, generator=g)
+    q, k = torch.randn(n, H * D, generator=g), torch.randn(n, G * D, generator=g)
+    v = torch.randn(n, G * Dv, generator=g)
     m = {"heads": H, "kv_heads": G, "dim": D, "vdim": Dv}
     one_q, one_k = torch.ones(H * D), torch.ones(G * D)
     qq, kk = plain.attention_inputs(q.double(), k.double(), one_q.double(), one_k.double(), m, 1e-6)
@@ -409,8 +414,8 @@ def _latent_case(g, n, H, R, window, spots):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("H,R,window", [(5, 40, 10), (3, 33, 37), (1, 16, 1), (9, 200, 0), (2, 600, 129)])
 def test_latent_attention_window_and_sink(device, H, R, window):
-    """The latent kernel with a window and a sink, no rotated part, through scattered pages and in portions: loud keys at
-    the first position, at page borders, on the window's edge and one outside it."""
+    """The latent kernel with a window and a sink, no rotated part, through scattered pages and in portions: loud keys
+    at the first position, at page borders, on the window's edge and one outside it."""
     g = torch.Generator().manual_seed(H + R)
     n = 150
     w = window or 10 ** 6
@@ -467,8 +472,8 @@ def test_latent_attention_matrix_cores_window_and_sink(H, R, window, n):
     for rows in (n - 40, 1, 38, 1):
         bt, ts, pos, sl = pg.step([(0, at, rows)])
         qd = torch.cat([torch.zeros(rows, H * 8), c[at:at + rows]], 1).to(dev).to(torch.bfloat16)
-        hops.latent_prep(qd, H, 8, 0, R, H * 8, torch.ones(R, dtype=torch.bfloat16, device=dev), 0.0, pos, None, 0, cache,
-                         sl, torch.empty(rows, H, 0, dtype=torch.bfloat16, device=dev), cache_t)
+        hops.latent_prep(qd, H, 8, 0, R, H * 8, torch.ones(R, dtype=torch.bfloat16, device=dev), 0.0, pos, None, 0,
+                         cache, sl, torch.empty(rows, H, 0, dtype=torch.bfloat16, device=dev), cache_t)
         tiles = torch.tensor([(a, min(tt, rows - a), 0, 0) for a in range(0, rows, tt)], dtype=torch.int32, device=dev)
         q = qb[:, at:at + rows].contiguous().to(dev)
         qr = torch.empty(rows, H, 0, dtype=torch.bfloat16, device=dev)

@@ -187,6 +187,42 @@ MOZIDRA_PRESETS: dict[str, dict] = {
 }
 
 
+def _magedra(width: int, heads: int, kv_heads: int, n_layers: int, vocab: int, ff: int, streams: int = 4,
+             head_dim: int = 128) -> dict:
+    """A Magedra config dict at transformer-like sizes: layers cycle latent attention (rank 512, rotated part 64,
+    query rank 3 x the latent's), minGRU (as wide as the model), parallel (grouped-query attention with a head mix
+    beside HGRN2 with ``width / 128`` heads of 64 x 128) and minGRU; every layer with a clamped dense feed-forward;
+    the second half of the depth runs the first half's tensors when the depth is a multiple of 8."""
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    kinds = []
+    for i in range(n_layers):
+        k = i % 4
+        if k == 0:
+            m = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536,
+                 "rot": {"base": 500000.0, "dims": 64}, "scale": (128 + 64) ** -0.5}
+            kinds.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+        elif k == 2:
+            left = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim,
+                    "rot": {"base": 100000.0, "dims": head_dim // 2}, "scale": head_dim ** -0.5}
+            right = {"heads": max(1, width // 128), "dim": 64, "vdim": 128}
+            kinds.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.7,
+                                                        "right_scale": 0.6}, "mlp": mlp})
+        else:
+            kinds.append({"type": "mingru", "mixer": {"width": width}, "mlp": mlp})
+    if n_layers % 8 == 0:
+        half = n_layers // 2
+        kinds = kinds[:half] + [dict(kinds[j], weights_of=j) for j in range(half)]
+    return {"architecture": "Magedra", "vocab": vocab, "width": width, "layers": kinds, "norm": {"eps": 1e-6},
+            "streams": streams, "residual_mult": 0.5, "logit_scale": 0.5}
+
+
+MAGEDRA_PRESETS: dict[str, dict] = {
+    # widths, heads and vocabularies of the Llama presets above (random init)
+    "magedra-small": _magedra(1024, 16, 2, 8, 128256, 3584),
+    "magedra-tiny": _magedra(512, 8, 2, 4, 32000, 1024, streams=2, head_dim=64),
+}
+
+
 def _budurax_config(c: dict, name: str):
     from kafka_llm_service_amd.models.budurax import BuduraxConfig
 
@@ -205,15 +241,23 @@ def _mozidra_config(c: dict, name: str):
     return MozidraConfig.from_dict(c, name=name)
 
 
+def _magedra_config(c: dict, name: str):
+    from kafka_llm_service_amd.models.magedra import MagedraConfig
+
+    return MagedraConfig.from_dict(c, name=name)
+
+
 # config.json "architecture" (lower case) -> config class of a model family that names itself there
-ARCH_CONFIGS = {"budurax": _budurax_config, "lisorax": _lisorax_config, "mozidra": _mozidra_config}
+ARCH_CONFIGS = {"budurax": _budurax_config, "lisorax": _lisorax_config, "mozidra": _mozidra_config,
+                "magedra": _magedra_config}
 # model families whose kernels are built for float32 as well as bfloat16 (EngineConfig.dtype)
-FP32_ARCHS = ("budurax", "lisorax", "mozidra")
+FP32_ARCHS = ("budurax", "lisorax", "mozidra", "magedra")
 
 
 def _from_json(path: Path):
     """A config.json names its model class: ``"architecture": "Budurax"`` (models/budurax.py), ``"Lisorax"``
-    (models/lisorax.py), ``"Mozidra"`` (models/mozidra.py), else HF Llama / Mixtral."""
+    (models/lisorax.py), ``"Mozidra"`` (models/mozidra.py), ``"Magedra"`` (models/magedra.py), else HF Llama /
+    Mixtral."""
     c = json.loads(path.read_text())
     make = ARCH_CONFIGS.get(str(c.get("architecture", "")).lower())
     if make is not None:
@@ -230,9 +274,11 @@ def get_config(name: str):
         return _lisorax_config(LISORAX_PRESETS[name], name)
     if name in MOZIDRA_PRESETS:
         return _mozidra_config(MOZIDRA_PRESETS[name], name)
+    if name in MAGEDRA_PRESETS:
+        return _magedra_config(MAGEDRA_PRESETS[name], name)
     p = Path(name)
     if p.is_dir() and (p / "config.json").exists():
         return _from_json(p / "config.json")
     if p.suffix == ".json" and p.exists():
         return _from_json(p)
-    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS) + sorted(BUDURAX_PRESETS) + sorted(LISORAX_PRESETS) + sorted(MOZIDRA_PRESETS)}")
+    raise KeyError(f"unknown model {name!r}; presets: {sorted(PRESETS) + sorted(BUDURAX_PRESETS) + sorted(LISORAX_PRESETS) + sorted(MOZIDRA_PRESETS) + sorted(MAGEDRA_PRESETS)}")

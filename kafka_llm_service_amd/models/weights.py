@@ -273,7 +273,7 @@ def build_model(cfg: ModelConfig, device, tp: int = 1, tp_rank: int = 0, seed: i
                 max_positions: int | None = None, dp_attention: tuple[int, int] | None = None, dtype=None):
     """``dp_attention = (ep, ep_rank)``: whole attention on this rank, experts sharded over the EP group.
     The model class follows ``cfg.arch`` (MODEL_CLASSES)."""
-    if cfg.arch in ("budurax", "lisorax", "mozidra"):  # segment-planned families: own tensor names, bf16 or fp32
+    if cfg.arch in ("budurax", "lisorax", "mozidra", "magedra"):  # segment-planned families: own tensor names
         if cfg.arch == "budurax":
             from kafka_llm_service_amd.models import budurax as fam
 
@@ -282,6 +282,10 @@ def build_model(cfg: ModelConfig, device, tp: int = 1, tp_rank: int = 0, seed: i
             from kafka_llm_service_amd.models import mozidra as fam
 
             cls = fam.MozidraLM
+        elif cfg.arch == "magedra":
+            from kafka_llm_service_amd.models import magedra as fam
+
+            cls = fam.MagedraLM
         else:
             from kafka_llm_service_amd.models import lisorax as fam
 

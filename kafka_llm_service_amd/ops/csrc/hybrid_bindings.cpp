@@ -80,7 +80,7 @@ hipError_t kafka_hy_mlstm_scan(int f32, const void* qkv, int64_t qs, const float
                                int64_t os, hipStream_t st);
 hipError_t kafka_hy_head_norm_gate(int f32, const float* o, int64_t os_, const void* w, const void* g, int64_t gs,
                                    int g_off, int H, int Dv, float eps, void* out, int64_t outs, int64_t T,
-                                   hipStream_t st);
+                                   float scale, hipStream_t st);
 int kafka_hy_router_max_e();
 int kafka_hy_router_max_k();
 hipError_t kafka_hy_moe_topk(const float* logits, int64_t ls, int E, int k, float* tw, int* te, int64_t T,
@@ -98,7 +98,7 @@ hipError_t kafka_hy_stream_step(float* xs, int64_t s_stride, int64_t t_stride, i
                                 int y_f32, const void* y2, int64_t y2s, int y2_f32, const float* row_scale,
                                 const float* mix, const float* wr, const float* rd, const float* nw, float eps,
                                 void* out, int64_t os, int out_f32, float* total, int64_t ts, int64_t T, int d,
-                                hipStream_t st);
+                                int center, hipStream_t st);
 hipError_t kafka_hy_swish_clamp_mul(int f32, const void* gu, int64_t gs, void* out, int64_t os, int64_t T, int F,
                                     float limit, float alpha, hipStream_t st);
 hipError_t kafka_hy_qk_norm_rope_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
@@ -111,17 +111,39 @@ int kafka_hy_window_attn_max_dv();
 hipError_t kafka_hy_window_attn(int f32, const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
                                 int bt_stride, const int* tok_seg, const int64_t* positions, int H, int G, int D,
                                 int Dv, float scale, int window, const float* sink, void* out, int64_t os, int64_t T,
-                                hipStream_t st);
+                                int shared_keys, hipStream_t st);
 int kafka_hy_window_attn_mfma_ok(int page, int D, int Dv, int rep);
 hipError_t kafka_hy_window_attn_mfma(const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
                                      int bt_stride, const int* items, int n_items, const int64_t* positions, int H,
                                      int G, int D, int Dv, float scale, int window, const float* sink, void* out,
-                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, hipStream_t st);
+                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, int shared_keys,
+                                     hipStream_t st);
 int kafka_hy_grouped_router_max_e();
 int kafka_hy_grouped_router_max_k();
 int kafka_hy_grouped_router_max_g();
 hipError_t kafka_hy_moe_topk_grouped(const float* logits, int64_t ls, int E, int k, const float* corr, int groups,
                                      int keep, float eps, float* tw, int* te, float* gate, int64_t T, hipStream_t st);
+
+// gated recurrences beside attention, rotation + head mix + paged store (hybrid_parallel.hip)
+hipError_t kafka_hy_act_norm(int f32, const void* x, int64_t xs, int c0, int n, const float* w, float eps, void* out,
+                             int64_t os, int64_t T, int center, hipStream_t st);
+hipError_t kafka_hy_gate_mul(int f32, const void* a, int64_t as, const void* g, int64_t gs, int g_off, float scale,
+                             void* out, int64_t os, int64_t T, int n, hipStream_t st);
+int kafka_hy_mingru_chunk();
+hipError_t kafka_hy_mingru_scan(int f32, const void* proj, int64_t ps, const float* bias, const int* seg, int R,
+                                float* state, void* out, int64_t os, int W, hipStream_t st);
+hipError_t kafka_hy_mingru_scan_chunked(int f32, const void* proj, int64_t ps, const float* bias, const int* seg, int R,
+                                        int nch, float* ab, float* ce, float* state, void* out, int64_t os, int64_t T,
+                                        int W, hipStream_t st);
+int kafka_hy_hgrn2_max_d();
+hipError_t kafka_hy_hgrn2_scan(int f32, const void* proj, int64_t ps, int q_off, int f_off, int v_off,
+                               const float* f_bias, const float* lower, int H, int D, int Dv, const int* seg, int R,
+                               float* S, float* out, int64_t os, hipStream_t st);
+int kafka_hy_rope_store_max_q();
+hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
+                                  const int64_t* positions, const float* cos_sin, int dims, int pairs,
+                                  const float* talk, void* kc, void* vt, const int64_t* slots, void* q_out, int64_t qos,
+                                  int64_t T, hipStream_t st);
 }
 
 namespace {
@@ -274,8 +296,9 @@ void latent_prep(at::Tensor qgd, int64_t H, int64_t dim, int64_t rd, int64_t R, 
   const int f32 = act_f32(qgd);
   same_act(f32, {&cache, &q_rot});
   const int64_t T = qgd.size(0);
-  // a model without a rotated part: rd = 0, dims = 0, no table
-  TORCH_CHECK(H > 0 && dim >= 0 && rd >= 0 && dim + rd > 0 && R > 0 && dims >= 0 && dims % 2 == 0 && dims <= rd &&
+  // a model without a rotated part: rd = 0, dims = 0, no table; H = 0: the queries come from elsewhere and only the
+  // cache row is written
+  TORCH_CHECK(H >= 0 && dim >= 0 && rd >= 0 && dim + rd > 0 && R > 0 && dims >= 0 && dims % 2 == 0 && dims <= rd &&
                   (dims > 0) == (rd > 0) && H * (dim + rd) <= qgd.size(1), "latent_prep: head sizes");
   TORCH_CHECK(cos_sin.has_value() == (dims > 0), "latent_prep: a rotation table comes with rot dims, and only then");
   TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
@@ -639,17 +662,22 @@ void mlstm_scan(at::Tensor qkv, at::Tensor gates, int64_t H, int64_t D, int64_t 
                              stream()));
 }
 
-void head_norm_gate(at::Tensor o, at::Tensor w, at::Tensor g, int64_t g_off, int64_t H, double eps, at::Tensor out) {
-  rows2d(o, "o"); rows2d(g, "g"); rows2d(out, "out"); f32t(o, "o");
+void head_norm_gate(at::Tensor o, at::Tensor w, OptT g, int64_t g_off, int64_t H, double eps, at::Tensor out,
+                    double scale) {
+  rows2d(o, "o"); rows2d(out, "out"); f32t(o, "o");
   const int f32 = act_f32(out);
-  same_act(f32, {&w, &g});
+  same_act(f32, {&w});
   const int64_t T = o.size(0), n = o.size(1);
   vec(w, n, "w");
-  TORCH_CHECK(H >= 1 && n % H == 0 && g.size(0) == T && g_off >= 0 && g_off + n <= g.size(1) && out.size(0) == T &&
-                  out.size(1) == n, "head_norm_gate: shapes");
-  HY_HIP(kafka_hy_head_norm_gate(f32, o.data_ptr<float>(), o.stride(0), w.data_ptr(), g.data_ptr(), g.stride(0),
-                                 (int)g_off, (int)H, (int)(n / H), (float)eps, out.data_ptr(), out.stride(0), T,
-                                 stream()));
+  TORCH_CHECK(H >= 1 && n % H == 0 && out.size(0) == T && out.size(1) == n, "head_norm_gate: shapes");
+  const void* gp = nullptr; int64_t gs = 0;
+  if (g.has_value()) {
+    rows2d(*g, "g"); same_act(f32, {&*g});
+    TORCH_CHECK(g->size(0) == T && g_off >= 0 && g_off + n <= g->size(1), "head_norm_gate: gate columns");
+    gp = g->data_ptr(); gs = g->stride(0);
+  }
+  HY_HIP(kafka_hy_head_norm_gate(f32, o.data_ptr<float>(), o.stride(0), w.data_ptr(), gp, gs, (int)g_off, (int)H,
+                                 (int)(n / H), (float)eps, out.data_ptr(), out.stride(0), T, (float)scale, stream()));
 }
 
 void moe_topk(at::Tensor logits, at::Tensor tw, at::Tensor te) {
@@ -720,7 +748,7 @@ const float* f32vec(const OptT& t, int64_t n, const char* name) {
 }
 
 void stream_step(at::Tensor xs, OptT y, OptT mix, OptT write, OptT read, OptT norm_w, double eps, OptT out, OptT y2,
-                 OptT row_scale, OptT total) {
+                 OptT row_scale, OptT total, bool center) {
   TORCH_CHECK(xs.is_cuda() && xs.scalar_type() == at::kFloat && xs.dim() == 3 && xs.stride(2) == 1,
               "stream_step: streams fp32 [S, T, d] with contiguous rows");
   const int64_t S = xs.size(0), T = xs.size(1), d = xs.size(2);
@@ -760,7 +788,7 @@ void stream_step(at::Tensor xs, OptT y, OptT mix, OptT write, OptT read, OptT no
   HY_HIP(kafka_hy_stream_step(xs.data_ptr<float>(), xs.stride(0), xs.stride(1), (int)S, yp, ys, yf, y2p, y2s, y2f,
                               f32vec(row_scale, T, "row_scale"), f32vec(mix, S * S, "mix"), f32vec(write, S, "write"),
                               f32vec(read, S, "read"), f32vec(norm_w, d, "norm_w"), (float)eps, op, os, of, tp, ts, T,
-                              (int)d, stream()));
+                              (int)d, center ? 1 : 0, stream()));
 }
 
 void swish_clamp_mul(at::Tensor gu, double limit, double alpha, at::Tensor out) {
@@ -815,15 +843,16 @@ void qk_norm_rope_store(at::Tensor qkv, int64_t H, int64_t G, int64_t D, int64_t
 }
 
 void window_attn(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor tok_seg, at::Tensor positions,
-                 int64_t H, int64_t G, double scale, int64_t window, OptT sink, at::Tensor out) {
+                 int64_t H, int64_t G, double scale, int64_t window, OptT sink, at::Tensor out, bool shared_keys) {
   rows2d(q, "q"); rows2d(out, "out");
   const int f32 = act_f32(q);
   same_act(f32, {&kc, &vt, &out});
   const int64_t T = q.size(0);
   TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && q.size(1) % H == 0 && out.size(0) == T && out.size(1) % H == 0,
               "window_attn: heads");
+  // shared_keys: a query row has the whole key row's size and meets all G key heads of a token
   const int64_t D = q.size(1) / H, Dv = out.size(1) / H;
-  paged_kv(kc, vt, G * D, G * Dv, "window_attn");
+  paged_kv(kc, vt, shared_keys ? D : G * D, G * Dv, "window_attn");
   TORCH_CHECK(D <= kafka_hy_window_attn_max_d() && Dv <= kafka_hy_window_attn_max_dv(), "window_attn: head sizes up to ",
               kafka_hy_window_attn_max_d(), " / ", kafka_hy_window_attn_max_dv());
   TORCH_CHECK(window >= 0, "window_attn: window");
@@ -834,14 +863,14 @@ void window_attn(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::
   HY_HIP(kafka_hy_window_attn(f32, q.data_ptr(), q.stride(0), kc.data_ptr(), vt.data_ptr(), bt.data_ptr<int>(),
                               (int)bt.stride(0), tok_seg.data_ptr<int>(), positions.data_ptr<int64_t>(), (int)H, (int)G,
                               (int)D, (int)Dv, (float)scale, (int)window, sink_ptr(sink, H), out.data_ptr(),
-                              out.stride(0), T, stream()));
+                              out.stride(0), T, shared_keys ? 1 : 0, stream()));
 }
 
 // the matrix-core kernel: items int32 [n, 4] = (first row, tokens, segment, 0), each at most 32 (token, query head of
 // one key/value head) rows of one segment
 void window_attn_mfma(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt, at::Tensor items, int64_t tile_tokens,
                       at::Tensor positions, int64_t H, int64_t G, double scale, int64_t window, OptT sink,
-                      at::Tensor out, int64_t nsplit, OptT po, OptT pml) {
+                      at::Tensor out, int64_t nsplit, OptT po, OptT pml, bool shared_keys) {
   for (const at::Tensor* t : {&q, &kc, &vt, &out})
     TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kBFloat16, "window_attn_mfma: bf16 GPU tensors");
   rows2d(q, "q"); rows2d(out, "out");
@@ -849,7 +878,7 @@ void window_attn_mfma(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt,
   TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && q.size(1) % H == 0 && out.size(0) == T && out.size(1) % H == 0,
               "window_attn_mfma: heads");
   const int64_t D = q.size(1) / H, Dv = out.size(1) / H, rep = H / G;
-  paged_kv(kc, vt, G * D, G * Dv, "window_attn_mfma");
+  paged_kv(kc, vt, shared_keys ? D : G * D, G * Dv, "window_attn_mfma");
   TORCH_CHECK(kafka_hy_window_attn_mfma_ok(16, (int)D, (int)Dv, (int)rep), "window_attn_mfma: sizes not supported");
   // 16-byte loads: every query row start must be a multiple of 8 elements
   TORCH_CHECK(q.stride(0) % 8 == 0 && (reinterpret_cast<uintptr_t>(q.data_ptr()) & 15) == 0,
@@ -874,7 +903,7 @@ void window_attn_mfma(at::Tensor q, at::Tensor kc, at::Tensor vt, at::Tensor bt,
                                    (int)bt.stride(0), items.data_ptr<int>(), (int)items.size(0),
                                    positions.data_ptr<int64_t>(), (int)H, (int)G, (int)D, (int)Dv, (float)scale,
                                    (int)window, sink_ptr(sink, H), out.data_ptr(), out.stride(0), (int)nsplit, pop,
-                                   pmlp, T, stream()));
+                                   pmlp, T, shared_keys ? 1 : 0, stream()));
 }
 
 void moe_topk_grouped(at::Tensor logits, int64_t E, at::Tensor corr, int64_t groups, int64_t keep, double eps,
@@ -895,6 +924,102 @@ void moe_topk_grouped(at::Tensor logits, int64_t E, at::Tensor corr, int64_t gro
                                    f32vec(corr, E, "correction"), (int)groups, (int)keep, (float)eps,
                                    tw.data_ptr<float>(), te.data_ptr<int>(),
                                    const_cast<float*>(f32vec(gate, T, "gate")), T, stream()));
+}
+
+void act_norm(at::Tensor x, int64_t c0, int64_t n, at::Tensor w, double eps, at::Tensor out, bool center) {
+  rows2d(x, "x"); rows2d(out, "out"); f32t(w, "w");
+  const int f32 = act_f32(x);
+  same_act(f32, {&out});
+  const int64_t T = x.size(0);
+  vec(w, n, "w");
+  TORCH_CHECK(c0 >= 0 && n >= 1 && c0 + n <= x.size(1) && out.size(0) == T && out.size(1) == n, "act_norm: columns");
+  HY_HIP(kafka_hy_act_norm(f32, x.data_ptr(), x.stride(0), (int)c0, (int)n, w.data_ptr<float>(), (float)eps,
+                           out.data_ptr(), out.stride(0), T, center ? 1 : 0, stream()));
+}
+
+void gate_mul(at::Tensor a, at::Tensor g, int64_t g_off, double scale, at::Tensor out) {
+  rows2d(a, "a"); rows2d(g, "g"); rows2d(out, "out");
+  const int f32 = act_f32(a);
+  same_act(f32, {&g, &out});
+  const int64_t T = a.size(0), n = a.size(1);
+  TORCH_CHECK(g.size(0) == T && g_off >= 0 && g_off + n <= g.size(1) && out.size(0) == T && out.size(1) == n,
+              "gate_mul: shapes");
+  HY_HIP(kafka_hy_gate_mul(f32, a.data_ptr(), a.stride(0), g.data_ptr(), g.stride(0), (int)g_off, (float)scale,
+                           out.data_ptr(), out.stride(0), T, (int)n, stream()));
+}
+
+// (seg comes from the step plan, which keeps every segment's rows inside the step)
+void mingru_scan(at::Tensor proj, at::Tensor bias, int64_t W, at::Tensor seg, at::Tensor state, at::Tensor out,
+                 int64_t max_rows) {
+  rows2d(proj, "proj"); rows2d(out, "out"); f32t(bias, "bias"); f32t(state, "state");
+  const int f32 = act_f32(proj);
+  same_act(f32, {&out});
+  const int64_t T = proj.size(0);
+  seg_only(seg);
+  TORCH_CHECK(W >= 1 && proj.size(1) >= 3 * W && out.size(0) == T && out.size(1) == W, "mingru_scan: shapes");
+  vec(bias, 2 * W, "bias");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 2 && state.size(1) == W, "mingru_scan: state fp32 [slots, W]");
+  const int64_t R = seg.size(0), CH = kafka_hy_mingru_chunk();
+  if (max_rows > CH && R > 0) {
+    TORCH_CHECK(max_rows <= T, "mingru_scan: max_rows beyond the step's rows");
+    const int64_t nch = (max_rows + CH - 1) / CH;
+    auto ab = at::empty({T * 2 * W}, state.options());
+    auto ce = at::empty({R * nch * 2 * W}, state.options());
+    HY_HIP(kafka_hy_mingru_scan_chunked(f32, proj.data_ptr(), proj.stride(0), bias.data_ptr<float>(),
+                                        seg.data_ptr<int>(), (int)R, (int)nch, ab.data_ptr<float>(),
+                                        ce.data_ptr<float>(), state.data_ptr<float>(), out.data_ptr(), out.stride(0), T,
+                                        (int)W, stream()));
+    return;
+  }
+  HY_HIP(kafka_hy_mingru_scan(f32, proj.data_ptr(), proj.stride(0), bias.data_ptr<float>(), seg.data_ptr<int>(), (int)R,
+                              state.data_ptr<float>(), out.data_ptr(), out.stride(0), (int)W, stream()));
+}
+
+void hgrn2_scan(at::Tensor proj, int64_t q_off, int64_t f_off, int64_t v_off, at::Tensor f_bias, at::Tensor lower,
+                int64_t H, int64_t D, int64_t Dv, at::Tensor seg, at::Tensor S, at::Tensor out) {
+  rows2d(proj, "proj"); rows2d(out, "out"); f32t(f_bias, "f_bias"); f32t(lower, "lower"); f32t(S, "S"); f32t(out, "out");
+  const int f32 = act_f32(proj);
+  const int64_t T = proj.size(0), C = proj.size(1);
+  seg_only(seg);
+  TORCH_CHECK(H >= 1 && D >= 1 && Dv >= 1 && D <= kafka_hy_hgrn2_max_d(), "hgrn2_scan: head sizes (dim up to ",
+              kafka_hy_hgrn2_max_d(), ")");
+  TORCH_CHECK(q_off >= 0 && q_off + H * D <= C && f_off >= 0 && f_off + H * D <= C && v_off >= 0 &&
+                  v_off + H * Dv <= C && out.size(0) == T && out.size(1) == H * Dv, "hgrn2_scan: columns");
+  vec(f_bias, H * D, "f_bias"); vec(lower, H * D, "lower");
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 4 && S.size(1) == H && S.size(2) == D && S.size(3) == Dv,
+              "hgrn2_scan: state fp32 [slots, H, D, Dv]");
+  HY_HIP(kafka_hy_hgrn2_scan(f32, proj.data_ptr(), proj.stride(0), (int)q_off, (int)f_off, (int)v_off,
+                             f_bias.data_ptr<float>(), lower.data_ptr<float>(), (int)H, (int)D, (int)Dv,
+                             seg.data_ptr<int>(), (int)seg.size(0), S.data_ptr<float>(), out.data_ptr<float>(),
+                             out.stride(0), stream()));
+}
+
+void rope_kv_store(at::Tensor qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, at::Tensor positions, OptT cos_sin,
+                   int64_t dims, bool pairs, OptT talk, at::Tensor kc, at::Tensor vt, at::Tensor slots,
+                   at::Tensor q_out) {
+  rows2d(qkv, "qkv"); rows2d(q_out, "q_out");
+  const int f32 = act_f32(qkv);
+  same_act(f32, {&kc, &vt, &q_out});
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && qkv.size(1) >= H * D + G * D + G * Dv &&
+                  q_out.size(0) == T && q_out.size(1) == (talk.has_value() ? H * G * D : H * D),
+              "rope_kv_store: head sizes (q_out [T, H D], or [T, H G D] with a head mix)");
+  TORCH_CHECK(dims >= 0 && dims % 2 == 0 && dims <= D && cos_sin.has_value() == (dims > 0),
+              "rope_kv_store: rot dims even, at most the head size, with their table");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+                  positions.numel() == T && slots.is_cuda() && slots.scalar_type() == at::kLong &&
+                  slots.is_contiguous() && slots.numel() == T, "rope_kv_store: positions / slots int64 [T]");
+  if (dims > 0)
+    TORCH_CHECK(cos_sin->is_cuda() && cos_sin->scalar_type() == at::kFloat && cos_sin->is_contiguous() &&
+                    cos_sin->dim() == 2 && cos_sin->size(1) == dims, "rope_kv_store: cos_sin fp32 [positions, dims]");
+  TORCH_CHECK(!talk.has_value() || H * D <= kafka_hy_rope_store_max_q(), "rope_kv_store: a head mix takes up to ",
+              kafka_hy_rope_store_max_q(), " query values per row");
+  paged_kv(kc, vt, G * D, G * Dv, "rope_kv_store");
+  // positions index the table's rows and slots the cache on the device: the step plan keeps both in range
+  HY_HIP(kafka_hy_rope_kv_store(f32, qkv.data_ptr(), qkv.stride(0), (int)H, (int)G, (int)D, (int)Dv,
+                                positions.data_ptr<int64_t>(), dims > 0 ? cos_sin->data_ptr<float>() : nullptr,
+                                (int)dims, pairs ? 1 : 0, f32vec(talk, H * H, "head mix"), kc.data_ptr(), vt.data_ptr(),
+                                slots.data_ptr<int64_t>(), q_out.data_ptr(), q_out.stride(0), T, stream()));
 }
 
 }  // namespace
@@ -934,7 +1059,8 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_rglru_scan", &rglru_scan, py::arg("gates"), py::arg("proj"), py::arg("u"), py::arg("rate"), py::arg("seg"),
         py::arg("state"), py::arg("out"), py::arg("max_rows") = 0);
   m.def("hy_mlstm_scan", &mlstm_scan);
-  m.def("hy_head_norm_gate", &head_norm_gate);
+  m.def("hy_head_norm_gate", &head_norm_gate, py::arg("o"), py::arg("w"), py::arg("g"), py::arg("g_off"), py::arg("H"),
+        py::arg("eps"), py::arg("out"), py::arg("scale") = 1.0);
   m.def("hy_moe_topk", &moe_topk);
   m.def("hy_moe_rows", &moe_rows, py::arg("h"), py::arg("wgu"), py::arg("wd"), py::arg("tw"), py::arg("te"),
         py::arg("a"), py::arg("out"), py::arg("limit") = 0.0, py::arg("alpha") = 1.0);
@@ -943,17 +1069,25 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_stream_step", &stream_step, py::arg("xs"), py::arg("y") = py::none(), py::arg("mix") = py::none(),
         py::arg("write") = py::none(), py::arg("read") = py::none(), py::arg("norm_w") = py::none(),
         py::arg("eps") = 0.0, py::arg("out") = py::none(), py::arg("y2") = py::none(),
-        py::arg("row_scale") = py::none(), py::arg("total") = py::none());
+        py::arg("row_scale") = py::none(), py::arg("total") = py::none(), py::arg("center") = false);
   m.def("hy_swish_clamp_mul", &swish_clamp_mul);
   m.def("hy_qk_norm_rope_store", &qk_norm_rope_store);
-  m.def("hy_window_attn", &window_attn);
+  m.def("hy_window_attn", &window_attn, py::arg("q"), py::arg("kc"), py::arg("vt"), py::arg("bt"), py::arg("tok_seg"),
+        py::arg("positions"), py::arg("H"), py::arg("G"), py::arg("scale"), py::arg("window"), py::arg("sink"),
+        py::arg("out"), py::arg("shared_keys") = false);
   m.def("hy_window_attn_mfma_ok",
         [](int page, int D, int Dv, int rep) { return kafka_hy_window_attn_mfma_ok(page, D, Dv, rep) != 0; });
   m.def("hy_window_attn_mfma", &window_attn_mfma, py::arg("q"), py::arg("kc"), py::arg("vt"), py::arg("bt"),
         py::arg("items"), py::arg("tile_tokens"), py::arg("positions"), py::arg("H"), py::arg("G"), py::arg("scale"),
         py::arg("window"), py::arg("sink"), py::arg("out"), py::arg("nsplit") = 1, py::arg("po") = py::none(),
-        py::arg("pml") = py::none());
+        py::arg("pml") = py::none(), py::arg("shared_keys") = false);
   m.def("hy_moe_topk_grouped", &moe_topk_grouped);
+  m.def("hy_act_norm", &act_norm);
+  m.def("hy_gate_mul", &gate_mul);
+  m.def("hy_mingru_scan", &mingru_scan, py::arg("proj"), py::arg("bias"), py::arg("W"), py::arg("seg"),
+        py::arg("state"), py::arg("out"), py::arg("max_rows") = 0);
+  m.def("hy_hgrn2_scan", &hgrn2_scan);
+  m.def("hy_rope_kv_store", &rope_kv_store);
   m.def("hy_sigmoid_attn_mfma_ok",
         [](int page, int D, int Dv, int rep) { return kafka_hy_sigmoid_attn_mfma_ok(page, D, Dv, rep) != 0; });
   m.def("hy_sigmoid_attn_mfma", &sigmoid_attn_mfma, py::arg("q"), py::arg("q_off"), py::arg("kc"), py::arg("vt"),

@@ -616,7 +616,8 @@ template <typename AT>
 __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restrict__ o, int64_t os_,
                                                             const AT* __restrict__ w, const AT* __restrict__ g,
                                                             int64_t gs, int g_off, int H, int Dv, float eps,
-                                                            AT* __restrict__ out, int64_t outs, int64_t pairs) {
+                                                            AT* __restrict__ out, int64_t outs, int64_t pairs,
+                                                            float scale) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * (NT / 64) + wave;
   if (pair >= pairs) return;
@@ -628,7 +629,9 @@ __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restr
   const float rs = 1.0f / sqrtf(wave_sum(s) / (float)Dv + eps);
   for (int i = lane; i < Dv; i += 64) {
     const int c = h * Dv + i;
-    stf(out + t * outs + c, r[i] * rs * ldf(w + c) * sigmoidf(ldf(g + t * gs + g_off + c)));
+    float v = r[i] * rs * ldf(w + c) * scale;
+    if (g != nullptr) v *= sigmoidf(ldf(g + t * gs + g_off + c));
+    stf(out + t * outs + c, v);
   }
 }
 
@@ -931,13 +934,13 @@ hipError_t kafka_hy_mlstm_scan(int f32, const void* qkv, int64_t qs, const float
 
 hipError_t kafka_hy_head_norm_gate(int f32, const float* o, int64_t os_, const void* w, const void* g, int64_t gs,
                                    int g_off, int H, int Dv, float eps, void* out, int64_t outs, int64_t T,
-                                   hipStream_t st) {
+                                   float scale, hipStream_t st) {
   if (T <= 0) return hipSuccess;
   const int64_t pairs = T * H;
   const int grid = (int)((pairs + NT / 64 - 1) / (NT / 64));
   DISPATCH_AT(f32, {
     head_norm_gate_kernel<AT><<<grid, NT, 0, st>>>(o, os_, (const AT*)w, (const AT*)g, gs, g_off, H, Dv, eps, (AT*)out,
-                                                   outs, pairs);
+                                                   outs, pairs, scale);
   });
   return hipGetLastError();
 }

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
                                                          const float* __restrict__ mix, const float* __restrict__ wr,
                                                          const float* __restrict__ rd, const float* __restrict__ nw,
                                                          float eps, void* __restrict__ out, int64_t os, bool out_f32,
-                                                         float* __restrict__ total, int64_t ts, int d) {
+                                                         float* __restrict__ total, int64_t ts, int d, bool center) {
   constexpr int NV = stream_nv(S);
   __shared__ float red[NT / 64];
   __shared__ float cM[SMAX * SMAX], cb[SMAX], ca[SMAX];
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
     return u;
   };
   float xv[NV][S], yv[NV];
-  float acc = 0.f;
+  float acc = 0.f, accs = 0.f;   // sum of squares and plain sum of the read values
   // the register part: every load of the row's first NT * NV columns is issued before anything is stored
 #pragma unroll
   for (int it = 0; it < NV; ++it) {
@@ -124,6 +124,7 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
       if (rd != nullptr) {
         const float u = read(xv[it]);
         acc += u * u;
+        accs += u;
         yv[it] = u;  // (the sublayer output is used up: its register keeps the read value)
       }
     }
@@ -148,12 +149,31 @@ __global__ __launch_bounds__(NT) void stream_step_kernel(float* __restrict__ xs,
     if (rd != nullptr) {
       const float u = read(x);
       acc += u * u;
+      accs += u;
     }
   }
   if (rd == nullptr) return;
+  // a centred norm takes the row's mean off first and measures the deviations in a second pass over the read values
+  float mean = 0.f;
+  if (center) {
+    mean = block_sum<NT>(accs, red) / (float)d;
+    acc = 0.f;
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int i = threadIdx.x + it * NT;
+      if (i < d) acc += (yv[it] - mean) * (yv[it] - mean);
+    }
+    for (int i = threadIdx.x + NV * NT; i < d; i += NT) {
+      float x[S];
+#pragma unroll
+      for (int s = 0; s < S; ++s) x[s] = xr[s * s_stride + i];
+      const float u = read(x) - mean;
+      acc += u * u;
+    }
+  }
   const float rs = 1.0f / sqrtf(block_sum<NT>(acc, red) / (float)d + eps);
   auto store = [&](int i, float u) {
-    const float v = u * rs * nw[i];
+    const float v = (u - mean) * rs * nw[i];
     if (out_f32) reinterpret_cast<float*>(out)[t * os + i] = v;
     else reinterpret_cast<bf16*>(out)[t * os + i] = (bf16)v;
   };
@@ -232,7 +252,7 @@ __global__ __launch_bounds__(NT) void qk_norm_rope_store_kernel(
 }
 
 // ---- windowed softmax attention with a sink -----------------------------------------------------------------------
-constexpr int WA_MAXD = 512;  // query / key size (the query row sits in LDS as fp32)
+constexpr int WA_MAXD = 1024;  // query / key size (the query row sits in LDS as fp32)
 constexpr int WA_NV = 8;      // value size up to 64 * WA_NV
 
 template <typename AT>
@@ -241,9 +261,11 @@ __global__ __launch_bounds__(NT) void window_attn_kernel(const AT* __restrict__ 
                                                          const int* __restrict__ bt, int bt_stride,
                                                          const int* __restrict__ tok_seg,
                                                          const int64_t* __restrict__ positions, int H, int G, int D,
-                                                         int Dv, float scale_log2e, int window,
+                                                         int Dv, int Ck, int kstep, float scale_log2e, int window,
                                                          const float* __restrict__ sink, AT* __restrict__ out,
                                                          int64_t os, int64_t pairs) {
+  // D: size of a query row and of the key it meets; key/value head g's key starts at column g * kstep of a key row of
+  // Ck columns (kstep = D: one key head per key/value head; kstep = 0, D = Ck: every query row meets the whole key row)
   __shared__ float qsh[NT / 64][WA_MAXD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * (NT / 64) + wave;
@@ -258,7 +280,7 @@ __global__ __launch_bounds__(NT) void window_attn_kernel(const AT* __restrict__ 
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int Ck = G * D, Cv = G * Dv;
+  const int Cv = G * Dv;
   float acc[WA_NV];
 #pragma unroll
   for (int i = 0; i < WA_NV; ++i) acc[i] = 0.f;
@@ -273,7 +295,7 @@ __global__ __launch_bounds__(NT) void window_attn_kernel(const AT* __restrict__ 
     const int64_t j = j0 + lane;
     float s = -INFINITY;
     if (j <= p && j >= lo) {
-      const AT* kr = kc + ((int64_t)pages[j / PAGE] * PAGE + (j % PAGE)) * Ck + (int64_t)g * D;
+      const AT* kr = kc + ((int64_t)pages[j / PAGE] * PAGE + (j % PAGE)) * Ck + (int64_t)g * kstep;
       float dot = 0.f;
       for (int i = 0; i < D; ++i) dot += qw[i] * ldf(kr + i);
       s = dot;
@@ -336,8 +358,9 @@ template <int TW, int NKSC>
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     const bf16* __restrict__ q, int64_t qs, const bf16* __restrict__ kc, const bf16* __restrict__ vt,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ items, const int64_t* __restrict__ positions,
-    int H, int G, int D, int Dv, float scale_log2e, int window, const float* __restrict__ sink,
+    int H, int G, int D, int Dv, int Ck, int kstep, float scale_log2e, int window, const float* __restrict__ sink,
     bf16* __restrict__ out, int64_t os, float* __restrict__ po, float* __restrict__ pml, int64_t T) {
+  // (D, Ck, kstep as in window_attn_kernel: kstep = 0 and D = Ck when every query row meets the whole key row)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int nks = D >> 4, qstride = D + 8;
   bf16* Qs = reinterpret_cast<bf16*>(smem);                       // [32][D + 8]
@@ -372,14 +395,14 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[tw][i] = 0.f;
   const int* btr = bt + (int64_t)sg * bt_stride;
-  const int Ck = G * D, Cv = G * Dv;
+  const int Cv = G * Dv;
   const int nblocks = (maxpos >> 7) + 1;
   const int kbmin = window > 0 ? max(0, (int)positions[t0] - window + 1) >> 7 : 0;
   const bf16* qrow = Qs + lr * qstride + 8 * lh;
   bf16x8 kf[NKSC];
   auto fetch_keys = [&](int kb) {
     const int kcix = min(kb * 128 + 32 * w + lr, maxpos);  // past the tile's last position: a valid row, masked below
-    const bf16* krow = kc + ((int64_t)btr[kcix >> 4] * PAGE + (kcix & 15)) * Ck + (int64_t)g * D + 8 * lh;
+    const bf16* krow = kc + ((int64_t)btr[kcix >> 4] * PAGE + (kcix & 15)) * Ck + (int64_t)g * kstep + 8 * lh;
 #pragma unroll
     for (int ks = 0; ks < NKSC; ++ks)
       if (ks < nks) kf[ks] = load_bf16x8(krow + 16 * ks);
@@ -660,12 +683,12 @@ hipError_t kafka_hy_stream_step(float* xs, int64_t s_stride, int64_t t_stride, i
                                 int y_f32, const void* y2, int64_t y2s, int y2_f32, const float* row_scale,
                                 const float* mix, const float* wr, const float* rd, const float* nw, float eps,
                                 void* out, int64_t os, int out_f32, float* total, int64_t ts, int64_t T, int d,
-                                hipStream_t st) {
+                                int center, hipStream_t st) {
   if (T <= 0 || d <= 0) return hipSuccess;
   if (S < 1 || S > SMAX) return hipErrorInvalidValue;
   auto a = [&](auto k) {
     k<<<(unsigned)T, NT, 0, st>>>(xs, s_stride, t_stride, y, ys, y_f32 != 0, y2, y2s, y2_f32 != 0, row_scale, mix, wr,
-                                  rd, nw, eps, out, os, out_f32 != 0, total, ts, d);
+                                  rd, nw, eps, out, os, out_f32 != 0, total, ts, d, center != 0);
   };
   switch (S) {
     case 1: a(stream_step_kernel<1>); break;
@@ -718,15 +741,17 @@ int kafka_hy_window_attn_max_dv() { return 64 * WA_NV; }
 hipError_t kafka_hy_window_attn(int f32, const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
                                 int bt_stride, const int* tok_seg, const int64_t* positions, int H, int G, int D,
                                 int Dv, float scale, int window, const float* sink, void* out, int64_t os, int64_t T,
-                                hipStream_t st) {
+                                int shared_keys, hipStream_t st) {
+  // shared_keys: D is the whole key row's size and every query row meets all G key heads of a token at once
   if (T <= 0) return hipSuccess;
   if (D > WA_MAXD || Dv > 64 * WA_NV || G < 1 || H % G || window < 0) return hipErrorInvalidValue;
   const int64_t pairs = T * H;
   const int grid = (int)((pairs + NT / 64 - 1) / (NT / 64));
+  const int Ck = shared_keys ? D : G * D, kstep = shared_keys ? 0 : D;
   DISPATCH_AT(f32, {
     window_attn_kernel<AT><<<grid, NT, 0, st>>>((const AT*)q, qs, (const AT*)kc, (const AT*)vt, bt, bt_stride, tok_seg,
-                                                positions, H, G, D, Dv, scale * LOG2E, window, sink, (AT*)out, os,
-                                                pairs);
+                                                positions, H, G, D, Dv, Ck, kstep, scale * LOG2E, window, sink,
+                                                (AT*)out, os, pairs);
   });
   return hipGetLastError();
 }
@@ -739,15 +764,17 @@ int kafka_hy_window_attn_mfma_ok(int page, int D, int Dv, int rep) {
 hipError_t kafka_hy_window_attn_mfma(const void* q, int64_t qs, const void* kc, const void* vt, const int* bt,
                                      int bt_stride, const int* items, int n_items, const int64_t* positions, int H,
                                      int G, int D, int Dv, float scale, int window, const float* sink, void* out,
-                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, hipStream_t st) {
+                                     int64_t os, int nsplit, float* po, float* pml, int64_t T, int shared_keys,
+                                     hipStream_t st) {
   if (n_items <= 0) return hipSuccess;
+  const int Ck = shared_keys ? D : G * D, kstep = shared_keys ? 0 : D;
   if (G < 1 || H % G || window < 0 || !kafka_hy_window_attn_mfma_ok(PAGE, D, Dv, H / G)) return hipErrorInvalidValue;
   if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (po == nullptr || pml == nullptr))) return hipErrorInvalidValue;
   const size_t lds = (size_t)WM_ROWS * (D + 8) * 2 + WM_ROWS * 136 * 2 + 5 * WM_ROWS * 4;
   const dim3 grid((unsigned)n_items, (unsigned)G, (unsigned)nsplit);
   auto a = [&](auto k) {
     k<<<grid, 256, lds, st>>>((const bf16*)q, qs, (const bf16*)kc, (const bf16*)vt, bt, bt_stride, items, positions, H,
-                              G, D, Dv, scale * LOG2E, window, sink, (bf16*)out, os, po, pml, T);
+                              G, D, Dv, Ck, kstep, scale * LOG2E, window, sink, (bf16*)out, os, po, pml, T);
   };
   const int nks = D / 16, tw = ((Dv + 31) / 32 + 3) / 4;
   if (tw == 1 && nks <= 4) a(window_attn_mfma_kernel<1, 4>);

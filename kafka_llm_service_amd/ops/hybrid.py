@@ -342,12 +342,13 @@ def mlstm_scan(qkv, gates, H: int, D: int, Dv: int, cap: float, tok_seg, seg, S,
         ref.mlstm_scan(qkv, gates, H, D, Dv, cap, tok_seg, seg, S, nrm, mx, out)
 
 
-def head_norm_gate(o, w, g, g_off: int, H: int, eps, out) -> None:
-    """out = o / rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) for o fp32 [T, H Dv]."""
+def head_norm_gate(o, w, g, g_off: int, H: int, eps, out, scale: float = 1.0) -> None:
+    """out = o / rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) * scale for o fp32 [T, H Dv]; ``g`` None:
+    no gate. ``out`` may be a column slice of a wider buffer."""
     if _gpu(o):
-        ext().hy_head_norm_gate(o, w, g, int(g_off), int(H), float(eps), out)
+        ext().hy_head_norm_gate(o, w, g, int(g_off), int(H), float(eps), out, float(scale))
     else:
-        ref.head_norm_gate(o, w, g, g_off, H, eps, out)
+        ref.head_norm_gate(o, w, g, g_off, H, eps, out, scale)
 
 
 def moe_router(h, w, b, k: int):
@@ -451,13 +452,14 @@ STREAM_MAX = 16   # residual streams the stream kernel takes
 
 
 def stream_step(xs, y=None, mix=None, write=None, read=None, norm_w=None, eps=0.0, out=None, y2=None,
-                row_scale=None, total=None) -> None:
+                row_scale=None, total=None, center: bool = False) -> None:
     """One pass over the residual streams xs fp32 [S, T, d] (hyper-connections), every part optional:
       write   with ``mix`` fp32 [S, S] (indexed [from, to]) and ``write`` fp32 [S]: all streams at once from the old
               ones, xs[r] <- sum_s mix[s, r] xs[s] + write[r] * (y + row_scale[:, None] * y2); y / y2 [T, d] in the
               activation dtype or fp32, row_scale fp32 [T] (y2 and row_scale come together or not at all);
       read    with ``read`` fp32 [S] and ``norm_w`` fp32 [d] (a one-plus weight is passed as 1 + w): out = u /
-              sqrt(mean(u^2) + eps) * norm_w for u = sum_s read[s] xs[s] of the NEW streams, in out's dtype;
+              sqrt(mean(u^2) + eps) * norm_w for u = sum_s read[s] xs[s] of the NEW streams, in out's dtype; with
+              ``center`` the row's mean is taken off u first (a layer norm with a weight and no bias);
       total   fp32 [T, d] <- sum_s xs[s] of the new streams.
     All arithmetic is fp32. A plain residual is S = 1 with mix = write = read = 1."""
     S = xs.shape[0]
@@ -470,9 +472,9 @@ def stream_step(xs, y=None, mix=None, write=None, read=None, norm_w=None, eps=0.
     if (read is None) != (norm_w is None) or (read is None) != (out is None):
         raise ValueError("stream_step: a read needs read, norm_w and out")
     if _gpu(xs):
-        ext().hy_stream_step(xs, y, mix, write, read, norm_w, float(eps), out, y2, row_scale, total)
+        ext().hy_stream_step(xs, y, mix, write, read, norm_w, float(eps), out, y2, row_scale, total, bool(center))
     else:
-        ref.stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total)
+        ref.stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total, center)
 
 
 def swish_clamp_mul(gu, limit: float, alpha: float, out) -> None:
@@ -506,19 +508,20 @@ def qk_norm_rope_store(qkv, H: int, G: int, D: int, Dv: int, q_w, k_w, eps, posi
                                lam, k_cache, v_cache_t, slot_mapping, q_out)
 
 
-def window_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int) -> bool:
+def window_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int, shared_keys: bool = False) -> bool:
     """bf16 GPU tensors of sizes the matrix-core kernel takes (16-token pages, key size a multiple of 16, sizes up
-    to 256, at most 32 query heads per key/value head, 16-byte aligned query rows)."""
+    to 256, at most 32 query heads per key/value head, 16-byte aligned query rows). With ``shared_keys`` the key size
+    is the whole key row's."""
     if not (q.is_cuda and q.dtype == torch.bfloat16):
         return False
     if q.stride(0) % 8 or q.data_ptr() % 16:  # query rows are read in 16-byte pieces
         return False
-    return bool(ext().hy_window_attn_mfma_ok(k_cache.shape[1], k_cache.shape[2] // G, v_cache_t.shape[1] // G,
-                                             H // G))
+    return bool(ext().hy_window_attn_mfma_ok(k_cache.shape[1], k_cache.shape[2] // (1 if shared_keys else G),
+                                             v_cache_t.shape[1] // G, H // G))
 
 
 def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int, G: int, scale: float, window: int,
-                sink, out, tiles=None, max_keys: int = 0) -> None:
+                sink, out, tiles=None, max_keys: int = 0, shared_keys: bool = False) -> None:
     """Causal softmax attention over paged keys [pages, page, G D] and page-wise transposed values [pages, G Dv, page]:
     row t at position p, head h (key/value head h // (H / G)) sees the keys p - window < j <= p (window 0: all j <= p);
         out = sum_j e^(s_j) v_j / (sum_j e^(s_j) + e^(sink[h])),  s_j = (q . k_j) scale
@@ -526,11 +529,14 @@ def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int,
     (int32 [n, 4] = (first row, tokens, segment, 0), at most ``sig_tile_tokens(H, G)`` tokens of one segment each) and
     sizes it takes, bf16 runs on the matrix cores; else one wave per (row, head) on the vector units, keys in order,
     whatever the batch. ``max_keys`` (the step's longest context) lets a launch of few tiles split its key ranges
-    over more workgroups (``sig_splits``); a merge pass combines them."""
+    over more workgroups (``sig_splits``); a merge pass combines them.
+    ``shared_keys``: q is [T, H G D] - every query head is a row of the whole key row's size and its score is the
+    product with ALL G key heads of a token (queries that hold a mix over the heads, see ``rope_kv_store``); values
+    stay per key/value head."""
     if window < 0:
         raise ValueError("window_attn: window must be positive (0 = every earlier position)")
     if _gpu(q):
-        if tiles is not None and window_attn_mfma_ok(q, k_cache, v_cache_t, H, G):
+        if tiles is not None and window_attn_mfma_ok(q, k_cache, v_cache_t, H, G, shared_keys):
             tt = sig_tile_tokens(H, G)
             if window and max_keys:  # a tile's key range is at most the window and its own tokens long
                 max_keys = min(max_keys, window + tt)
@@ -540,12 +546,13 @@ def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int,
                 po = torch.empty(ns, q.shape[0], out.shape[1], dtype=torch.float32, device=q.device)
                 pml = torch.empty(ns, q.shape[0], H, 2, dtype=torch.float32, device=q.device)
             ext().hy_window_attn_mfma(q, k_cache, v_cache_t, block_tables, tiles, tt, positions, int(H), int(G),
-                                      float(scale), int(window), sink, out, ns, po, pml)
+                                      float(scale), int(window), sink, out, ns, po, pml, bool(shared_keys))
         else:
             ext().hy_window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, int(H), int(G), float(scale),
-                                 int(window), sink, out)
+                                 int(window), sink, out, bool(shared_keys))
     else:
-        ref.window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out)
+        ref.window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out,
+                        shared_keys)
 
 
 def moe_router_grouped(h, w, correction, k: int, groups: int, keep: int, eps: float = 0.0, extra_gate: bool = False):
@@ -572,3 +579,75 @@ def moe_router_grouped(h, w, correction, k: int, groups: int, keep: int, eps: fl
     else:
         ref.moe_router_grouped(h, w, E, correction, k, groups, keep, eps, tw, te, gate)
     return tw, te, gate
+
+
+# ---- gated recurrences beside attention (minGRU, HGRN2), rotation + head mix + paged store --------------------------
+def act_norm(x, c0: int, n: int, w, eps, out, center: bool = False) -> None:
+    """out [T, n] = norm(x[:, c0 : c0 + n]) * w over rows of activations (x in the activation dtype or fp32, w fp32
+    [n]): an RMS norm, or with ``center`` a layer norm with a weight and no bias. Statistics in fp32."""
+    if c0 < 0 or c0 + n > x.shape[1]:
+        raise ValueError("act_norm: columns outside the row")
+    if _gpu(x):
+        ext().hy_act_norm(x, int(c0), int(n), w, float(eps), out, bool(center))
+    else:
+        ref.act_norm(x, c0, n, w, eps, out, center)
+
+
+def gate_mul(a, g, g_off: int, scale: float, out) -> None:
+    """out = a * sigmoid(g[:, g_off : g_off + n]) * scale for a [T, n]; ``out`` may be a column slice."""
+    if _gpu(a):
+        ext().hy_gate_mul(a, g, int(g_off), float(scale), out)
+    else:
+        ref.gate_mul(a, g, g_off, scale, out)
+
+
+def mingru_scan(proj, bias, W: int, tok_seg, seg, state, out, max_rows: int = 0) -> None:
+    """minGRU over a step's segments: a gated recurrence whose gates read only the current token. proj [T, >= 3 W] =
+    pre-activations of the update gate | the candidate | the output gate, bias fp32 [2 W] for the first two:
+        z = sigmoid(p_z + b_z);  u = p_x + b_x;  c = u + 1/2 where u >= 0, sigmoid(u) where u < 0;
+        S <- (1 - z) S + z c;  out = S silu(p_g).
+    state fp32 [slots, W], zero before a sequence's first token (the slot is then written, not read). Gates, the
+    candidate and the state are fp32. ``max_rows``: an upper bound of the longest segment's rows when the caller
+    knows one: long segments run in chunks (per-chunk scans from zero with the chunk's decay product, entry states
+    carried in order, a second pass from the entry states), which re-associates the sums - fp32 rounding only."""
+    if _gpu(proj):
+        ext().hy_mingru_scan(proj, bias, int(W), seg, state, out, int(max_rows))
+    else:
+        ref.mingru_scan(proj, bias, W, tok_seg, seg, state, out)
+
+
+def hgrn2_scan(proj, q_off: int, f_off: int, v_off: int, f_bias, lower, H: int, D: int, Dv: int, tok_seg, seg, S,
+               out) -> None:
+    """HGRN2 over a step's segments: linear attention whose forget gate is also (one minus) its key. proj [T, ...]
+    holds the raw queries (H D columns at q_off), raw forget gates (H D at f_off) and values (H Dv at v_off);
+    f_bias, lower fp32 [H D]. Per head:
+        f = lower + (1 - lower) sigmoid(p_f + b_f);  S <- diag(f) S + (1 - f) v^T;  out = S^T silu(p_q).
+    S fp32 [slots, H, D, Dv], zero before a sequence's first token; out fp32 [T, H Dv]."""
+    if _gpu(proj):
+        ext().hy_hgrn2_scan(proj, int(q_off), int(f_off), int(v_off), f_bias, lower, int(H), int(D), int(Dv), seg, S,
+                            out)
+    else:
+        ref.hgrn2_scan(proj, q_off, f_off, v_off, f_bias, lower, H, D, Dv, tok_seg, seg, S, out)
+
+
+def rope_kv_store(qkv, H: int, G: int, D: int, Dv: int, positions, cos_sin, rot_dims: int, pairs: bool, talk,
+                  k_cache, v_cache_t, slot_mapping, q_out) -> None:
+    """Attention inputs from the fused projection row [q (H D) | k (G D) | v (G Dv)] (further columns are ignored):
+      * rotation of the first ``rot_dims`` dimensions of every q and k head by the row's position (``cos_sin`` fp32
+        [positions, rot_dims] = cos | sin per frequency): dimension i with i + rot_dims / 2, or with ``pairs``
+        dimension 2i with 2i + 1; rot_dims = 0 and no table: no rotation;
+      * k -> k_cache [pages, page, G D] at the row's slot; v -> v_cache_t [pages, G Dv, page];
+      * q -> q_out [T, H D]; or with ``talk`` fp32 [H, H] (scores mixed over the heads before the softmax,
+        s'_h = sum_g talk[h, g] s_g) -> q_out [T, H G D]: q'[h] = for every key head c the sum over its query heads g
+        of talk[h, g] q[g], so that q'[h] . (the whole key row) = s'_h (``window_attn`` with ``shared_keys``).
+    Rotation and the mix are fp32."""
+    if rot_dims % 2 or rot_dims > D or (rot_dims > 0) != (cos_sin is not None):
+        raise ValueError("rope_kv_store: rot_dims even, at most the head size, with its table")
+    if G < 1 or H % G:
+        raise ValueError("rope_kv_store: query heads must split evenly over the key heads")
+    if _gpu(qkv):
+        ext().hy_rope_kv_store(qkv, int(H), int(G), int(D), int(Dv), positions, cos_sin, int(rot_dims), bool(pairs),
+                               talk, k_cache, v_cache_t, slot_mapping, q_out)
+    else:
+        ref.rope_kv_store(qkv, H, G, D, Dv, positions, cos_sin, rot_dims, pairs, talk, k_cache, v_cache_t,
+                          slot_mapping, q_out)

@@ -266,12 +266,16 @@ def mlstm_scan(qkv, gates, H, D, Dv, cap, tok_seg, seg, S, nrm, mx, out):
         S[slot], nrm[slot], mx[slot] = Ss, ns, ms
 
 
-def head_norm_gate(o, w, g, g_off, H, eps, out):
-    """out = unit_rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) (o fp32 [T, H Dv])."""
+def head_norm_gate(o, w, g, g_off, H, eps, out, scale=1.0):
+    """out = unit_rms_per_head(o) * w * sigmoid(g[:, g_off : g_off + H Dv]) * scale (o fp32 [T, H Dv]; no gate
+    when ``g`` is None)."""
     T, n = o.shape
     v = o.float().view(T, H, n // H)
     v = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps)
-    out.copy_(v.reshape(T, n) * w.float() * torch.sigmoid(g[:, g_off:g_off + n].float()))
+    v = v.reshape(T, n) * w.float()
+    if g is not None:
+        v = v * torch.sigmoid(g[:, g_off:g_off + n].float())
+    out.copy_((v * scale).to(out.dtype))
 
 
 def moe_router(h, w, b, k, topk_w, topk_e):
@@ -311,8 +315,9 @@ def add2(x, y1, y2=None):
     x += s
 
 
-def stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total):
-    """xs fp32 [S, T, d]: optional write (all streams from the old ones), optional normed read, optional sum."""
+def stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total, center=False):
+    """xs fp32 [S, T, d]: optional write (all streams from the old ones), optional normed read (RMS norm, or with
+    ``center`` a layer norm without bias), optional sum."""
     if mix is not None:
         ys = y.float()
         if y2 is not None:
@@ -321,6 +326,8 @@ def stream_step(xs, y, mix, write, read, norm_w, eps, out, y2, row_scale, total)
         xs.copy_(new)
     if read is not None:
         u = torch.einsum("s,std->td", read.float(), xs)
+        if center:
+            u = u - u.mean(-1, keepdim=True)
         out.copy_((u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * norm_w.float()).to(out.dtype))
     if total is not None:
         total.copy_(xs.sum(0))
@@ -352,7 +359,10 @@ def qk_norm_rope_store(qkv, H, G, D, Dv, q_w, k_w, eps, positions, cos_sin, rot_
     kv_store(torch.cat([k.reshape(T, Ck), v], 1).to(k_cache.dtype), 0, Ck, k_cache, v_cache_t, slot_mapping)
 
 
-def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out):
+def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, scale, window, sink, out,
+                shared_keys=False):
+    """``shared_keys``: every query head is a row of the whole key row's size and meets all G key heads at once
+    (queries that already hold a mix over the heads); values stay per key/value head."""
     T = q.shape[0]
     page, D = k_cache.shape[1], k_cache.shape[2] // G
     Dv = v_cache_t.shape[1] // G
@@ -363,8 +373,10 @@ def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H, G, s
         lo = max(0, n - window) if window else 0
         k = k_cache[pages].reshape(-1, G, D)[lo:n].float()                       # [n, G, D]
         v = v_cache_t[pages].permute(0, 2, 1).reshape(-1, G, Dv)[lo:n].float()   # [n, G, Dv]
-        qt = q[t].float().view(H, D)
-        s = torch.einsum("hd,jhd->hj", qt, k.repeat_interleave(rep, 1)) * scale
+        if shared_keys:
+            s = torch.einsum("hc,jc->hj", q[t].float().view(H, G * D), k.reshape(-1, G * D)) * scale
+        else:
+            s = torch.einsum("hd,jhd->hj", q[t].float().view(H, D), k.repeat_interleave(rep, 1)) * scale
         if sink is not None:
             s = torch.cat([s, sink.float()[:, None]], 1)
         pw = torch.softmax(s, -1)[:, :n - lo]
@@ -388,3 +400,83 @@ def moe_router_grouped(h, w, E, correction, k, groups, keep, eps, topk_w, topk_e
     topk_w.copy_(wv / (wv.sum(-1, keepdim=True) + eps))
     if gate is not None:
         gate.copy_(torch.sigmoid(z[:, E]))
+
+
+# ---- gated recurrences beside attention: minGRU, HGRN2; rotation + head mix + paged store ---------------------------
+def act_norm(x, c0, n, w, eps, out, center=False):
+    """out = norm(x[:, c0 : c0 + n]) * w: RMS norm, or with ``center`` a layer norm without bias."""
+    u = x[:, c0:c0 + n].float()
+    if center:
+        u = u - u.mean(-1, keepdim=True)
+    out.copy_((u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * w.float()).to(out.dtype))
+
+
+def gate_mul(a, g, g_off, scale, out):
+    """out = a * sigmoid(g[:, g_off : g_off + n]) * scale."""
+    n = a.shape[1]
+    out.copy_((a.float() * torch.sigmoid(g[:, g_off:g_off + n].float()) * scale).to(out.dtype))
+
+
+def mingru_scan(proj, bias, Wd, tok_seg, seg, state, out):
+    """proj [T, >= 3 W] = pre-activations of the update gate | the candidate | the output gate, bias fp32 [2 W] for
+    the first two: z = sigmoid(.), c = u + 1/2 where u >= 0 else sigmoid(u), S <- (1 - z) S + z c,
+    out = S silu(g); state fp32 [slots, W]."""
+    z = torch.sigmoid(proj[:, :Wd].float() + bias[:Wd].float())
+    u = proj[:, Wd:2 * Wd].float() + bias[Wd:].float()
+    c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = proj[:, 2 * Wd:3 * Wd].float()
+    y = g * torch.sigmoid(g)
+    for q0, n, p0, slot in seg.tolist():
+        S = state[slot].clone() if p0 > 0 else torch.zeros(Wd)
+        for t in range(q0, q0 + n):
+            S = (1.0 - z[t]) * S + z[t] * c[t]
+            out[t] = (S * y[t]).to(out.dtype)
+        state[slot] = S
+
+
+def hgrn2_scan(proj, q_off, f_off, v_off, f_bias, lower, H, D, Dv, tok_seg, seg, S, out):
+    """Per head: f = lower + (1 - lower) sigmoid(raw f + bias) per key channel, S <- diag(f) S + (1 - f) v^T,
+    out = S^T silu(raw q). proj [T, ...] holds raw q (H D) at q_off, raw f (H D) at f_off, v (H Dv) at v_off;
+    S fp32 [slots, H, D, Dv]; out fp32 [T, H Dv]."""
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * D].float()
+    q = (q * torch.sigmoid(q)).view(T, H, D)
+    lo = lower.float()
+    f = (lo + (1.0 - lo) * torch.sigmoid(proj[:, f_off:f_off + H * D].float() + f_bias.float())).view(T, H, D)
+    v = proj[:, v_off:v_off + H * Dv].float().view(T, H, Dv)
+    for q0, n, p0, slot in seg.tolist():
+        St = S[slot].clone() if p0 > 0 else torch.zeros(H, D, Dv)
+        for t in range(q0, q0 + n):
+            St = f[t][:, :, None] * St + (1.0 - f[t])[:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", St, q[t]).reshape(-1)
+        S[slot] = St
+
+
+def rope_kv_store(qkv, H, G, D, Dv, positions, cos_sin, rot_dims, pairs, talk, k_cache, v_cache_t, slot_mapping,
+                  q_out):
+    """Fused projection row [q (H D) | k (G D) | v (G Dv)]: rotation of the first rot_dims dimensions of every q and
+    k head (partners i, i + rot_dims / 2, or with ``pairs`` 2i, 2i + 1), keys and values into their pages. With
+    ``talk`` fp32 [H, H] the queries leave as q'[h] = [sum over the heads g of key head c of talk[h, g] q[g]] for
+    c = 0 .. G - 1 (row size G D): q'[h] . (whole key row) is the head-mixed score."""
+    T = qkv.shape[0]
+    Cq, Ck, Cv = H * D, G * D, G * Dv
+    q, k, v = (t.float() for t in qkv[:, :Cq + Ck + Cv].split([Cq, Ck, Cv], 1))
+    q, k = q.view(T, H, D).clone(), k.view(T, G, D).clone()
+    if rot_dims:
+        half = rot_dims // 2
+        cs = cos_sin[positions.long()]
+        c, s = cs[:, None, :half], cs[:, None, half:]
+        for x in (q, k):
+            if pairs:
+                a, b = x[..., 0:rot_dims:2].clone(), x[..., 1:rot_dims:2].clone()
+                x[..., 0:rot_dims:2] = a * c - b * s
+                x[..., 1:rot_dims:2] = b * c + a * s
+            else:
+                a, b = x[..., :half].clone(), x[..., half:rot_dims].clone()
+                x[..., :half] = a * c - b * s
+                x[..., half:rot_dims] = b * c + a * s
+    if talk is not None:
+        rep = H // G
+        q = torch.einsum("hcr,tcrd->thcd", talk.float().view(H, G, rep), q.view(T, G, rep, D)).reshape(T, H * Ck)
+    q_out.copy_(q.reshape(T, -1).to(q_out.dtype))
+    kv_store(torch.cat([k.reshape(T, Ck), v], 1).to(k_cache.dtype), 0, Ck, k_cache, v_cache_t, slot_mapping)

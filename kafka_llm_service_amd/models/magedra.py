@@ -523,8 +523,10 @@ class MagedraLM:
         xsel = xs.index_select(1, inp.logit_rows)
         hf = torch.empty(xsel.shape[1], d, dtype=dt, device=dev)
         hops.stream_step(xsel, read=self.sum_in, norm_w=self.final_norm, eps=eps, out=hf, center=True)
-        logits = self._lin(hf, self.head, getattr(self, "head_t", None)).float()[:, :cfg.vocab_size]
-        return logits * cfg.logit_scale if cfg.logit_scale != 1.0 else logits
+        logits = self._lin(hf, self.head, getattr(self, "head_t", None)).float()
+        if cfg.logit_scale != 1.0:
+            logits.mul_(cfg.logit_scale)
+        return logits[:, :cfg.vocab_size]   # (a view: the padded row stride is what the sampler reads)
 
     def _max_rows(self, m: SegMeta) -> int:
         return int(m.seg_host[:, 1].max()) if m.seg_host is not None and len(m.seg_host) else 0

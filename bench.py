@@ -107,7 +107,9 @@ def parse(argv=None):
                     help="model families to measure, of budurax, llama, lisorax (sigmoid attention, rglru, mlstm "
                          "layers with 8 routed experts, 2 per token, of half the dense feed-forward each), mozidra "
                          "(windowed latent and grouped-query attention over 4 residual streams; 8 group-routed "
-                         "experts, 2 per token, and a shared one, of a third of the dense feed-forward each)")
+                         "experts, 2 per token, and a shared one, of a third of the dense feed-forward each), magedra "
+                         "(latent attention, minGRU and parallel head-mixed attention + HGRN2 layers over 4 residual "
+                         "streams, the dense clamped feed-forward)")
     return ap.parse_args(argv)
 
 
@@ -118,7 +120,8 @@ def arch_compare(args) -> int:
     import torch
 
     from kafka_llm_service_amd.engine.engine import EngineConfig, LLMEngine
-    from kafka_llm_service_amd.models.config import ModelConfig, _budurax, _lisorax, _mozidra
+    from kafka_llm_service_amd.models.config import ModelConfig, _budurax, _lisorax, _magedra, _mozidra
+    from kafka_llm_service_amd.models.magedra import MagedraConfig
     from kafka_llm_service_amd.models.budurax import BuduraxConfig
     from kafka_llm_service_amd.models.lisorax import LisoraxConfig
     from kafka_llm_service_amd.models.mozidra import MozidraConfig
@@ -134,6 +137,8 @@ def arch_compare(args) -> int:
                                                name=f"lisorax-w{w}-l{L}"),
             "mozidra": MozidraConfig.from_dict(_mozidra(w, heads, max(1, heads // 4), L, vocab, ff // 3 // 256 * 256),
                                                name=f"mozidra-w{w}-l{L}"),
+            # (two key heads of 128: the head-mixed queries meet a 256-wide key row, the matrix-core kernel's limit)
+            "magedra": MagedraConfig.from_dict(_magedra(w, heads, 2, L, vocab, ff), name=f"magedra-w{w}-l{L}"),
             "llama": ModelConfig(name=f"llama-w{w}-l{L}", hidden_size=w, intermediate_size=ff, num_layers=L,
                                  num_heads=heads, num_kv_heads=max(1, heads // 4), vocab_size=vocab,
                                  max_position_embeddings=131072, bos_token_id=1, eos_token_ids=[2])}

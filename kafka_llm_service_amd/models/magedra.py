@@ -53,6 +53,7 @@ import math
 from dataclasses import dataclass, field
 from pathlib import Path
 
+import numpy as np
 import torch
 import torch.nn.functional as F
 
@@ -531,6 +532,21 @@ class MagedraLM:
     def _max_rows(self, m: SegMeta) -> int:
         return int(m.seg_host[:, 1].max()) if m.seg_host is not None and len(m.seg_host) else 0
 
+    def _chunk_plan(self, m: SegMeta, work: int):
+        """Device chunk tables of this step for a scan with ``work`` workgroups per segment (built once per step), None
+        = the plain scan fills the GPU or the segments are short."""
+        key = ("chunks", work)
+        if key not in m.cache:
+            p = hops.scan_chunks(m.seg_host, work)
+            if p is not None:
+                fresh, cont, cs, mx = p
+                up = torch.from_numpy(np.concatenate([fresh.reshape(-1), cont.reshape(-1),
+                                                      cs.reshape(-1)])).to(self.device)
+                a, b = fresh.size, fresh.size + cont.size
+                p = (up[:a].view(-1, 4), up[a:b].view(-1, 4), up[b:].view(-1, 4), mx)
+            m.cache[key] = p
+        return m.cache[key]
+
     def _mingru(self, lw, h, m: SegMeta, st: dict) -> torch.Tensor:
         Wd = int(lw.m["width"])
         proj = self._lin(h, lw.w_in, getattr(lw, "w_in_t", None))                 # [update gate | candidate | gate]
@@ -555,8 +571,13 @@ class MagedraLM:
         both = torch.empty(T, H * Dv + Hr * Dvr, dtype=dt, device=dev)            # [left heads | right heads]
         hops.gate_mul(ao, proj, lw.g_off, lw.left_scale, both[:, :H * Dv])
         o = torch.empty(T, Hr * Dvr, dtype=torch.float32, device=dev)
-        hops.hgrn2_scan(proj, lw.rq_off, lw.rf_off, lw.rv_off, lw.f_bias, lw.lower, Hr, Dr, Dvr, m.tok_seg, m.seg,
-                        st["S"], o)
+        plan = self._chunk_plan(m, Hr * -(-Dvr // 64)) if dev.type == "cuda" else None
+        if plan is not None:  # long prompt portions, few sequences: chunk-parallel scan
+            hops.hgrn2_scan_chunked(proj, lw.rq_off, lw.rf_off, lw.rv_off, lw.f_bias, lw.lower, Hr, Dr, Dvr, plan,
+                                    st["S"], o)
+        else:
+            hops.hgrn2_scan(proj, lw.rq_off, lw.rf_off, lw.rv_off, lw.f_bias, lw.lower, Hr, Dr, Dvr, m.tok_seg, m.seg,
+                            st["S"], o)
         hops.head_norm_gate(o, lw.rnorm, None, 0, Hr, self.cfg.norm_eps, both[:, H * Dv:], lw.right_scale)
         return self._lin(both, lw.o, getattr(lw, "o_t", None))
 

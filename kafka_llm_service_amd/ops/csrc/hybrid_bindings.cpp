@@ -139,6 +139,10 @@ int kafka_hy_hgrn2_max_d();
 hipError_t kafka_hy_hgrn2_scan(int f32, const void* proj, int64_t ps, int q_off, int f_off, int v_off,
                                const float* f_bias, const float* lower, int H, int D, int Dv, const int* seg, int R,
                                float* S, float* out, int64_t os, hipStream_t st);
+hipError_t kafka_hy_hgrn2_decay(int f32, const void* proj, int64_t ps, int f_off, const float* f_bias,
+                                const float* lower, int HD, const int* vseg, int n_chunks, float* F, hipStream_t st);
+hipError_t kafka_hy_hgrn2_combine(const int* cs, int R, const float* F, int HD, int Dv, float* tmp, float* state,
+                                  hipStream_t st);
 int kafka_hy_rope_store_max_q();
 hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
                                   const int64_t* positions, const float* cos_sin, int dims, int pairs,
@@ -1012,14 +1016,39 @@ void rope_kv_store(at::Tensor qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
   if (dims > 0)
     TORCH_CHECK(cos_sin->is_cuda() && cos_sin->scalar_type() == at::kFloat && cos_sin->is_contiguous() &&
                     cos_sin->dim() == 2 && cos_sin->size(1) == dims, "rope_kv_store: cos_sin fp32 [positions, dims]");
-  TORCH_CHECK(!talk.has_value() || H * D <= kafka_hy_rope_store_max_q(), "rope_kv_store: a head mix takes up to ",
-              kafka_hy_rope_store_max_q(), " query values per row");
+  TORCH_CHECK(!talk.has_value() || (H * D <= kafka_hy_rope_store_max_q() && H <= 64), "rope_kv_store: a head mix takes "
+              "up to 64 heads and ", kafka_hy_rope_store_max_q(), " query values per row");
   paged_kv(kc, vt, G * D, G * Dv, "rope_kv_store");
   // positions index the table's rows and slots the cache on the device: the step plan keeps both in range
   HY_HIP(kafka_hy_rope_kv_store(f32, qkv.data_ptr(), qkv.stride(0), (int)H, (int)G, (int)D, (int)Dv,
                                 positions.data_ptr<int64_t>(), dims > 0 ? cos_sin->data_ptr<float>() : nullptr,
                                 (int)dims, pairs ? 1 : 0, f32vec(talk, H * H, "head mix"), kc.data_ptr(), vt.data_ptr(),
                                 slots.data_ptr<int64_t>(), q_out.data_ptr(), q_out.stride(0), T, stream()));
+}
+
+// the chunk tables come from ops.hybrid.scan_chunks, which keeps chunks inside their segments and numbers them 0 .. n - 1
+void hgrn2_chunk_decay(at::Tensor proj, int64_t f_off, at::Tensor f_bias, at::Tensor lower, at::Tensor vseg,
+                       at::Tensor F) {
+  rows2d(proj, "proj"); f32t(f_bias, "f_bias"); f32t(lower, "lower"); f32t(F, "F");
+  seg_only(vseg);
+  const int64_t HD = lower.numel();
+  vec(f_bias, HD, "f_bias");
+  TORCH_CHECK(lower.is_contiguous() && f_off >= 0 && f_off + HD <= proj.size(1) && F.is_contiguous() &&
+                  F.numel() == vseg.size(0) * HD, "hgrn2_chunk_decay: shapes");
+  HY_HIP(kafka_hy_hgrn2_decay(act_f32(proj), proj.data_ptr(), proj.stride(0), (int)f_off, f_bias.data_ptr<float>(),
+                              lower.data_ptr<float>(), (int)HD, vseg.data_ptr<int>(), (int)vseg.size(0),
+                              F.data_ptr<float>(), stream()));
+}
+
+void hgrn2_chunk_combine(at::Tensor cs, at::Tensor F, at::Tensor tmp, at::Tensor state) {
+  seg_only(cs); f32t(F, "F"); f32t(tmp, "tmp"); f32t(state, "state");
+  TORCH_CHECK(tmp.is_contiguous() && tmp.dim() == 4 && state.is_contiguous() && state.dim() == 4 &&
+                  tmp.size(1) == state.size(1) && tmp.size(2) == state.size(2) && tmp.size(3) == state.size(3) &&
+                  F.is_contiguous() && F.numel() == tmp.size(0) * tmp.size(1) * tmp.size(2),
+              "hgrn2_chunk_combine: tmp [chunks, H, D, Dv], state [slots, H, D, Dv], F [chunks, H D]");
+  HY_HIP(kafka_hy_hgrn2_combine(cs.data_ptr<int>(), (int)cs.size(0), F.data_ptr<float>(),
+                                (int)(tmp.size(1) * tmp.size(2)), (int)tmp.size(3), tmp.data_ptr<float>(),
+                                state.data_ptr<float>(), stream()));
 }
 
 }  // namespace
@@ -1087,6 +1116,8 @@ void kafka_bind_hybrid(pybind11::module_& m) {
   m.def("hy_mingru_scan", &mingru_scan, py::arg("proj"), py::arg("bias"), py::arg("W"), py::arg("seg"),
         py::arg("state"), py::arg("out"), py::arg("max_rows") = 0);
   m.def("hy_hgrn2_scan", &hgrn2_scan);
+  m.def("hy_hgrn2_chunk_decay", &hgrn2_chunk_decay);
+  m.def("hy_hgrn2_chunk_combine", &hgrn2_chunk_combine);
   m.def("hy_rope_kv_store", &rope_kv_store);
   m.def("hy_sigmoid_attn_mfma_ok",
         [](int page, int D, int Dv, int rep) { return kafka_hy_sigmoid_attn_mfma_ok(page, D, Dv, rep) != 0; });

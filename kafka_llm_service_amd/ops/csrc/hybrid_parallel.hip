@@ -308,6 +308,48 @@ __global__ __launch_bounds__(NT) void hgrn2_scan_kernel(const AT* __restrict__ p
   }
 }
 
+// Chunk-parallel form for long segments, around two runs of the kernel above over the chunks as segments of their own:
+// hgrn2_decay: F[chunk][h D + d] = the product of the chunk's forget gates; hgrn2_combine: per segment, over its chunks
+// in order, tmp[chunk] (the chunk's scan from zero) is replaced by the chunk's entry state and the running state
+// becomes diag(F) state + local; the last one is the sequence's new state.
+template <typename AT>
+__global__ void hgrn2_decay_kernel(const AT* __restrict__ proj, int64_t ps, int f_off, const float* __restrict__ f_bias,
+                                   const float* __restrict__ lower, int HD, const int* __restrict__ vseg,
+                                   float* __restrict__ F) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= HD) return;
+  const int ch = blockIdx.y;
+  const int q0 = vseg[4 * ch], n = vseg[4 * ch + 1];
+  const float lo = lower[c], fb = f_bias[c];
+  float a = 1.f;
+  for (int j0 = 0; j0 < n; j0 += 8) {   // eight rows' gates requested together
+    float p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p[j] = ldf(proj + ((int64_t)q0 + min(j0 + j, n - 1)) * ps + f_off + c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j0 + j < n) a *= lo + (1.0f - lo) * sigmoidf(p[j] + fb);
+  }
+  F[(int64_t)ch * HD + c] = a;
+}
+
+__global__ void hgrn2_combine_kernel(const int* __restrict__ cs, const float* __restrict__ F, int HD, int Dv,
+                                     float* __restrict__ tmp, float* __restrict__ state) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (h, d, v) of the head matrices
+  const int64_t n = (int64_t)HD * Dv;
+  if (e >= n) return;
+  const int r = blockIdx.y;
+  const int first = cs[4 * r], cnt = cs[4 * r + 1], p0 = cs[4 * r + 2], slot = cs[4 * r + 3];
+  const int hd = (int)(e / Dv);
+  float S = p0 > 0 ? state[(int64_t)slot * n + e] : 0.f;
+  for (int c = first; c < first + cnt; ++c) {
+    const float L = tmp[(int64_t)c * n + e];
+    tmp[(int64_t)c * n + e] = S;
+    S = F[(int64_t)c * HD + hd] * S + L;
+  }
+  state[(int64_t)slot * n + e] = S;
+}
+
 // ---- attention inputs: rotation, head mix, paged store -------------------------------------------------------------------
 // One workgroup per row of the fused projection [q (H D) | k (G D) | v (G Dv) | ...]. With `talk` the rotated queries
 // wait in LDS (fp32) and leave as q'[h][c D + i] = sum_r talk[h][c rep + r] q[c rep + r][i] (rep = H / G).
@@ -316,54 +358,75 @@ __global__ __launch_bounds__(NT) void rope_kv_store_kernel(
     const AT* __restrict__ qkv, int64_t qs, int H, int G, int D, int Dv, const int64_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int dims, bool pairs, const float* __restrict__ talk, AT* __restrict__ kc,
     AT* __restrict__ vt, const int64_t* __restrict__ slots, AT* __restrict__ q_out, int64_t qos) {
-  extern __shared__ float qsh[];   // [H D] when the queries are mixed
+  extern __shared__ float qsh[];   // [H D] rotated queries, then [H H] mix weights, when the queries are mixed
   const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int Cq = H * D, Ck = G * D, Cv = G * Dv;
   const AT* row = qkv + t * qs;
   const int half = dims >> 1;
   const float* cs = dims > 0 ? cos_sin + positions[t] * dims : nullptr;
   const int64_t slot = slots[t];
-  // element i of a projection, rotated with its partner when it lies in a head's first `dims` dimensions
-  auto elem = [&](const AT* src, int i) {
-    const float a = ldf(src + i);
-    const int dh = i % D;
+  // dimension dh of the head that starts at `src`, rotated with its partner when it lies in the first `dims`
+  auto elem = [&](const AT* src, int dh) {
+    const float a = ldf(src + dh);
     if (dh >= dims) return a;
     int f, ip;
     bool second;
     if (pairs) {
       f = dh >> 1;
       second = dh & 1;
-      ip = second ? i - 1 : i + 1;
+      ip = second ? dh - 1 : dh + 1;
     } else {
       second = dh >= half;
       f = second ? dh - half : dh;
-      ip = second ? i - half : i + half;
+      ip = second ? dh - half : dh + half;
     }
     const float b = ldf(src + ip);
     const float c = cs[f], s = cs[half + f];
     return second ? a * c + b * s : a * c - b * s;
   };
-  for (int i = threadIdx.x; i < Cq; i += NT) {
-    const float v = elem(row, i);
-    if (talk != nullptr) qsh[i] = v;
-    else stf(q_out + t * qos + i, v);
-  }
+  // a wave per head, lanes over the head's dimensions (no index arithmetic per element)
+  for (int h = wave; h < H; h += NT / 64)
+    for (int dh = lane; dh < D; dh += 64) {
+      const float v = elem(row + h * D, dh);
+      if (talk != nullptr) qsh[h * D + dh] = v;
+      else stf(q_out + t * qos + h * D + dh, v);
+    }
   if (slot >= 0) {
     AT* kd = kc + slot * Ck;
-    for (int i = threadIdx.x; i < Ck; i += NT) stf(kd + i, elem(row + Cq, i));
+    for (int g = wave; g < G; g += NT / 64)
+      for (int dh = lane; dh < D; dh += 64) stf(kd + g * D + dh, elem(row + Cq + g * D, dh));
     AT* vd = vt + (slot / PAGE) * (int64_t)Cv * PAGE + (slot % PAGE);
     for (int i = threadIdx.x; i < Cv; i += NT) stf(vd + (int64_t)i * PAGE, ldf(row + Cq + Ck + i));
   }
   if (talk == nullptr) return;
+  float* tsh = qsh + Cq;
+  for (int i = threadIdx.x; i < H * H; i += NT) tsh[i] = talk[i];
   __syncthreads();
+  // a wave per (head h, key head c): its rep mix weights are wave-uniform, lanes run over the key head's dimensions
   const int rep = H / G;
-  for (int o = threadIdx.x; o < H * Ck; o += NT) {
-    const int h = o / Ck, rem = o - h * Ck, c = rem / D, i = rem - c * D;
-    const float* tr = talk + h * H + c * rep;
-    const float* qp = qsh + (c * rep) * D + i;
-    float v = 0.f;
-    for (int r = 0; r < rep; ++r) v += tr[r] * qp[r * D];
-    stf(q_out + t * qos + o, v);
+  for (int hc = wave; hc < H * G; hc += NT / 64) {
+    const int h = hc / G, c = hc - h * G;
+    const float* tr = tsh + h * H + c * rep;
+    for (int i = lane; i < D; i += 64) {
+      const float* qp = qsh + (c * rep) * D + i;
+      float v0 = 0.f, v1 = 0.f;
+      for (int r0 = 0; r0 < rep; r0 += 8) {   // eight weights and eight query values requested before the first use
+        float tv[8], qv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int r = min(r0 + j, rep - 1);
+          tv[j] = r0 + j < rep ? tr[r] : 0.f;
+          qv[j] = qp[r * D];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          v0 += tv[j] * qv[j];
+          v1 += tv[j + 1] * qv[j + 1];
+        }
+      }
+      stf(q_out + t * qos + (int64_t)hc * D + i, v0 + v1);
+    }
   }
 }
 
@@ -453,7 +516,25 @@ hipError_t kafka_hy_hgrn2_scan(int f32, const void* proj, int64_t ps, int q_off,
   return hipGetLastError();
 }
 
-int kafka_hy_rope_store_max_q() { return 12288; }   // H D floats of LDS when the queries are mixed
+hipError_t kafka_hy_hgrn2_decay(int f32, const void* proj, int64_t ps, int f_off, const float* f_bias,
+                                const float* lower, int HD, const int* vseg, int n_chunks, float* F, hipStream_t st) {
+  if (n_chunks <= 0 || HD <= 0) return hipSuccess;
+  if (n_chunks > 65535) return hipErrorInvalidValue;
+  const dim3 grid((HD + 63) / 64, n_chunks);
+  DISPATCH_AT(f32, { hgrn2_decay_kernel<AT><<<grid, 64, 0, st>>>((const AT*)proj, ps, f_off, f_bias, lower, HD, vseg, F); });
+  return hipGetLastError();
+}
+
+hipError_t kafka_hy_hgrn2_combine(const int* cs, int R, const float* F, int HD, int Dv, float* tmp, float* state,
+                                  hipStream_t st) {
+  if (R <= 0 || HD <= 0 || Dv <= 0) return hipSuccess;
+  if (R > 65535) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(((int64_t)HD * Dv + 255) / 256), R);
+  hgrn2_combine_kernel<<<grid, 256, 0, st>>>(cs, F, HD, Dv, tmp, state);
+  return hipGetLastError();
+}
+
+int kafka_hy_rope_store_max_q() { return 11264; }   // H D floats of LDS when the queries are mixed (+ H H <= 4096)
 
 hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
                                   const int64_t* positions, const float* cos_sin, int dims, int pairs,
@@ -461,8 +542,8 @@ hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, i
                                   int64_t T, hipStream_t st) {
   if (T <= 0) return hipSuccess;
   if (dims < 0 || dims % 2 || dims > D || (dims > 0 && cos_sin == nullptr) || G < 1 || H % G) return hipErrorInvalidValue;
-  if (talk != nullptr && H * D > kafka_hy_rope_store_max_q()) return hipErrorInvalidValue;
-  const size_t lds = talk != nullptr ? (size_t)H * D * sizeof(float) : 0;
+  if (talk != nullptr && (H * D > kafka_hy_rope_store_max_q() || H > 64)) return hipErrorInvalidValue;
+  const size_t lds = talk != nullptr ? (size_t)(H * D + H * H) * sizeof(float) : 0;
   DISPATCH_AT(f32, {
     rope_kv_store_kernel<AT><<<(unsigned)T, NT, lds, st>>>((const AT*)qkv, qs, H, G, D, Dv, positions, cos_sin, dims,
                                                            pairs != 0, talk, (AT*)kc, (AT*)vt, slots, (AT*)q_out, qos);

@@ -276,14 +276,14 @@ def sigmoid_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int) -> bool:
                                               H // G))
 
 
-def sig_splits(wgs: int, max_keys: int) -> int:
+def sig_splits(wgs: int, max_keys: int, target: int = ATTN_SPLIT_WGS) -> int:
     """Key-range splits of a matrix-core sigmoid attention launch: few workgroups (a decode step has one tile per
-    sequence and key/value head) against long contexts are dealt over more, each at least two 128-key blocks long; the
-    partial sums are added in order by a second launch."""
+    sequence and key/value head) against long contexts are dealt over more (up to ``target`` in all), each at least
+    two 128-key blocks long; the partial sums are added in order by a second launch."""
     blocks = -(-max_keys // 128)
-    if wgs >= ATTN_SPLIT_WGS // 2 or blocks < 4:
+    if wgs >= target // 2 or blocks < 4:
         return 1
-    return max(1, min(ATTN_SPLIT_MAX, ATTN_SPLIT_WGS // max(1, wgs), blocks // 2))
+    return max(1, min(ATTN_SPLIT_MAX, target // max(1, wgs), blocks // 2))
 
 
 def sigmoid_attn(q, q_off: int, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int, G: int, scale: float,
@@ -508,6 +508,9 @@ def qk_norm_rope_store(qkv, H: int, G: int, D: int, Dv: int, q_w, k_w, eps, posi
                                lam, k_cache, v_cache_t, slot_mapping, q_out)
 
 
+SHARED_SPLIT_WGS = 1024   # workgroups a shared-keys attention launch is split towards
+
+
 def window_attn_mfma_ok(q, k_cache, v_cache_t, H: int, G: int, shared_keys: bool = False) -> bool:
     """bf16 GPU tensors of sizes the matrix-core kernel takes (16-token pages, key size a multiple of 16, sizes up
     to 256, at most 32 query heads per key/value head, 16-byte aligned query rows). With ``shared_keys`` the key size
@@ -540,7 +543,9 @@ def window_attn(q, k_cache, v_cache_t, block_tables, tok_seg, positions, H: int,
             tt = sig_tile_tokens(H, G)
             if window and max_keys:  # a tile's key range is at most the window and its own tokens long
                 max_keys = min(max_keys, window + tt)
-            ns = sig_splits(tiles.shape[0] * G, max_keys) if max_keys else 1
+            # (shared keys: few key/value heads, every workgroup walks the whole key row - more, shorter ranges)
+            ns = sig_splits(tiles.shape[0] * G, max_keys, SHARED_SPLIT_WGS if shared_keys else ATTN_SPLIT_WGS) \
+                if max_keys else 1
             po = pml = None
             if ns > 1:
                 po = torch.empty(ns, q.shape[0], out.shape[1], dtype=torch.float32, device=q.device)
@@ -628,6 +633,24 @@ def hgrn2_scan(proj, q_off: int, f_off: int, v_off: int, f_bias, lower, H: int, 
                             out)
     else:
         ref.hgrn2_scan(proj, q_off, f_off, v_off, f_bias, lower, H, D, Dv, tok_seg, seg, S, out)
+
+
+def hgrn2_scan_chunked(proj, q_off: int, f_off: int, v_off: int, f_bias, lower, H: int, D: int, Dv: int, plan, S,
+                       out) -> None:
+    """The recurrence of ``hgrn2_scan`` in launches that expose more parallelism for long segments: every chunk
+    scanned from a zero state (and the product of its forget gates taken), the chunks' entry states rebuilt in order
+    (and the sequence's state advanced), every chunk scanned again from its entry state. ``plan``: device tensors
+    (vseg_fresh, vseg_cont, cs) + max chunks from ``scan_chunks``. Twice the arithmetic of the plain scan over
+    (chunks) times the workgroups; the result differs from the token-by-token order only by fp32 rounding (the entry
+    states are re-associated)."""
+    fresh, cont, cs, max_chunks = plan
+    tmp = torch.empty(fresh.shape[0], H, D, Dv, dtype=torch.float32, device=proj.device)
+    F = torch.empty(fresh.shape[0], H * D, dtype=torch.float32, device=proj.device)
+    e = ext()
+    e.hy_hgrn2_scan(proj, int(q_off), int(f_off), int(v_off), f_bias, lower, int(H), int(D), int(Dv), fresh, tmp, out)
+    e.hy_hgrn2_chunk_decay(proj, int(f_off), f_bias, lower, fresh, F)
+    e.hy_hgrn2_chunk_combine(cs, F, tmp, S)
+    e.hy_hgrn2_scan(proj, int(q_off), int(f_off), int(v_off), f_bias, lower, int(H), int(D), int(Dv), cont, tmp, out)
 
 
 def rope_kv_store(qkv, H: int, G: int, D: int, Dv: int, positions, cos_sin, rot_dims: int, pairs: bool, talk,

@@ -287,6 +287,51 @@ def test_hgrn2_scan_and_head_norm(device, H, D, Dv):
         assert close(got[s], want[s], 5e-5), s
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,D,Dv", [(3, 10, 14), (2, 64, 128), (1, 200, 70)])
+def test_hgrn2_scan_in_chunks(H, D, Dv):
+    """The chunk-parallel form (every chunk from zero, entry states carried in order, every chunk again) against the
+    token-by-token kernel and the plain function: two long segments, one of them continuing from a state."""
+    import numpy as np
+
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(D)
+    d, eps, n0, n1 = 24, 1e-5, 700, 513
+    W = {"q": torch.randn(H * D, d, generator=g) / 3, "f": torch.randn(H * D, d, generator=g) / 3,
+         "f.b": torch.randn(H * D, generator=g) + 2.0, "lower": torch.rand(H * D, generator=g) * 0.98,
+         "v": torch.randn(H * Dv, d, generator=g) / 3, "norm": torch.ones(Dv), "o": torch.eye(H * Dv)}
+    hs = [torch.randn(n0 + 40, d, generator=g), torch.randn(n1, d, generator=g)]
+    m = {"heads": H, "dim": D, "vdim": Dv}
+    want = [plain.hgrn2(h.double(), {k: v.double() for k, v in W.items()}, "", m, eps) for h in hs]
+    w_in = torch.cat([W["q"], W["f"], W["v"]], 0)
+    outs = []
+    for chunked in (False, True):
+        S = torch.full((2, H, D, Dv), float("nan"), device=dev)
+        got = [[], []]
+        for runs in ([(0, 0, 40)], [(0, 40, n0), (1, 0, n1)]):
+            rows = [(r0, n, p0, s) for (s, p0, n), r0 in zip(runs, np.cumsum([0] + [r[2] for r in runs])[:-1].tolist())]
+            ts, seg = seg_tensors(dev, rows)
+            proj = (torch.cat([hs[s][p0:p0 + n] for s, p0, n in runs]).double() @ w_in.double().T).float().to(dev)
+            o = torch.empty(proj.shape[0], H * Dv, device=dev)
+            args = (proj, 0, H * D, 2 * H * D, W["f.b"].to(dev), W["lower"].to(dev), H, D, Dv)
+            plan = hops.scan_chunks(np.asarray(rows, dtype=np.int32), H) if chunked else None
+            if plan is not None:
+                plan = tuple(torch.from_numpy(x).to(dev) for x in plan[:3]) + (plan[3],)
+                hops.hgrn2_scan_chunked(*args, plan, S, o)
+            else:
+                assert not chunked or len(runs) == 1
+                hops.hgrn2_scan(*args, ts, seg, S, o)
+            out = torch.empty_like(o)
+            hops.head_norm_gate(o, W["norm"].repeat(H).to(dev), None, 0, H, eps, out)
+            for (s, p0, n), (r0, _, _, _) in zip(runs, rows):
+                got[s].append(out[r0:r0 + n].cpu())
+        outs.append(([torch.cat(x) for x in got], S.cpu()))
+    for s in (0, 1):
+        assert close(outs[1][0][s], want[s], 5e-5), s
+        assert close(outs[1][0][s], outs[0][0][s], 5e-5), s
+    assert close(outs[1][1], outs[0][1], 5e-5)
+
+
 class Paged:
     """Scattered pages for sequences of given lengths, fed in given portions: the step tensors the kernels take."""
 
@@ -552,6 +597,19 @@ def test_long_prompt(bench_sharp, device):
     eng = bench_sharp.engine(device)
     assert rel_err(feed_all(eng, "a", t, [300]), bench_sharp.oracle(t)) < TOL["float32"]
     assert rel_err(feed_all(eng, "b", t, [129, 2, 100, 1]), bench_sharp.oracle(t)) < TOL["float32"]
+
+
+@pytest.mark.gpu
+def test_chunked_scans_in_the_engine(bench_sharp):
+    """A 700-token prompt beside a short one, then more of both: both recurrences take their chunked forms."""
+    t, u = toks(760, 211, 23), toks(30, 211, 24)
+    eng = bench_sharp.engine("cuda:0")
+    poison_state(eng)
+    a = eng.feed([("a", t[:20], list(range(20)))], [])
+    b = eng.feed([("a", t[20:720], list(range(700))), ("u", u[:9], list(range(9)))], [])
+    c = eng.feed([("u", u[9:], list(range(21))), ("a", t[720:], list(range(40)))], ["a", "u"])
+    assert rel_err(torch.cat([a, b[:700], c[21:]]), bench_sharp.oracle(t)) < TOL["float32"]
+    assert rel_err(torch.cat([b[700:], c[:21]]), bench_sharp.oracle(u)) < TOL["float32"]
 
 
 @pytest.mark.gpu

@@ -1016,8 +1016,9 @@ void rope_kv_store(at::Tensor qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
   if (dims > 0)
     TORCH_CHECK(cos_sin->is_cuda() && cos_sin->scalar_type() == at::kFloat && cos_sin->is_contiguous() &&
                     cos_sin->dim() == 2 && cos_sin->size(1) == dims, "rope_kv_store: cos_sin fp32 [positions, dims]");
-  TORCH_CHECK(!talk.has_value() || (H * D <= kafka_hy_rope_store_max_q() && H <= 64), "rope_kv_store: a head mix takes "
-              "up to 64 heads and ", kafka_hy_rope_store_max_q(), " query values per row");
+  TORCH_CHECK((H + G) * D + dims + (talk.has_value() ? H * H : 0) <= kafka_hy_rope_store_max_q(),
+              "rope_kv_store: q and k of a row, the rotation's table row and the head mix must fit ",
+              kafka_hy_rope_store_max_q(), " floats");
   paged_kv(kc, vt, G * D, G * Dv, "rope_kv_store");
   // positions index the table's rows and slots the cache on the device: the step plan keeps both in range
   HY_HIP(kafka_hy_rope_kv_store(f32, qkv.data_ptr(), qkv.stride(0), (int)H, (int)G, (int)D, (int)Dv,

@@ -351,81 +351,119 @@ __global__ void hgrn2_combine_kernel(const int* __restrict__ cs, const float* __
 }
 
 // ---- attention inputs: rotation, head mix, paged store -------------------------------------------------------------------
-// One workgroup per row of the fused projection [q (H D) | k (G D) | v (G Dv) | ...]. With `talk` the rotated queries
-// wait in LDS (fp32) and leave as q'[h][c D + i] = sum_r talk[h][c rep + r] q[c rep + r][i] (rep = H / G).
+// One workgroup per row of the fused projection [q (H D) | k (G D) | v (G Dv) | ...]. The row's q and k parts, the
+// position's cos | sin row and the mix matrix are staged in LDS as fp32 in one round of independent loads (a step of few
+// rows is one memory round trip per row); pairs are rotated in place (a thread owns both members); keys leave for
+// their page; the queries leave as they are, or with `talk` as q'[h][c D + i] = sum_r talk[h][c rep + r] q[c rep + r][i]
+// (rep = H / G).
+constexpr int MIX_REP = 32;   // query heads per key head whose values a lane keeps in registers for the head mix
+
 template <typename AT>
 __global__ __launch_bounds__(NT) void rope_kv_store_kernel(
     const AT* __restrict__ qkv, int64_t qs, int H, int G, int D, int Dv, const int64_t* __restrict__ positions,
     const float* __restrict__ cos_sin, int dims, bool pairs, const float* __restrict__ talk, AT* __restrict__ kc,
     AT* __restrict__ vt, const int64_t* __restrict__ slots, AT* __restrict__ q_out, int64_t qos) {
-  extern __shared__ float qsh[];   // [H D] rotated queries, then [H H] mix weights, when the queries are mixed
+  extern __shared__ float lds[];   // [H D + G D] q | k, [dims] cos | sin, [H H] mix weights
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int Cq = H * D, Ck = G * D, Cv = G * Dv;
   const AT* row = qkv + t * qs;
   const int half = dims >> 1;
-  const float* cs = dims > 0 ? cos_sin + positions[t] * dims : nullptr;
+  float* qk = lds;
+  float* cs = lds + Cq + Ck;
+  float* tsh = cs + dims;
   const int64_t slot = slots[t];
-  // dimension dh of the head that starts at `src`, rotated with its partner when it lies in the first `dims`
-  auto elem = [&](const AT* src, int dh) {
-    const float a = ldf(src + dh);
-    if (dh >= dims) return a;
-    int f, ip;
-    bool second;
-    if (pairs) {
-      f = dh >> 1;
-      second = dh & 1;
-      ip = second ? dh - 1 : dh + 1;
-    } else {
-      second = dh >= half;
-      f = second ? dh - half : dh;
-      ip = second ? dh - half : dh + half;
+  for (int i0 = 0; i0 < Cq + Ck; i0 += 8 * NT) {   // eight loads a thread in flight before the first LDS store
+    float tmp[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j * NT + threadIdx.x;
+      tmp[j] = i < Cq + Ck ? ldf(row + i) : 0.f;
     }
-    const float b = ldf(src + ip);
-    const float c = cs[f], s = cs[half + f];
-    return second ? a * c + b * s : a * c - b * s;
-  };
-  // a wave per head, lanes over the head's dimensions (no index arithmetic per element)
-  for (int h = wave; h < H; h += NT / 64)
-    for (int dh = lane; dh < D; dh += 64) {
-      const float v = elem(row + h * D, dh);
-      if (talk != nullptr) qsh[h * D + dh] = v;
-      else stf(q_out + t * qos + h * D + dh, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j * NT + threadIdx.x;
+      if (i < Cq + Ck) qk[i] = tmp[j];
     }
+  }
+  if (dims > 0) {
+    const float* src = cos_sin + positions[t] * dims;
+    for (int i = threadIdx.x; i < dims; i += NT) cs[i] = src[i];
+  }
+  if (talk != nullptr)
+    for (int i = threadIdx.x; i < H * H; i += NT) tsh[i] = talk[i];
+  if (slot >= 0) {
+    AT* vd = vt + (slot / PAGE) * (int64_t)Cv * PAGE + (slot % PAGE);
+#pragma unroll 4
+    for (int i = threadIdx.x; i < Cv; i += NT) vd[(int64_t)i * PAGE] = row[Cq + Ck + i];
+  }
+  __syncthreads();
+  // a wave per head (query heads, then key heads), lanes over its frequencies
+  for (int hd = wave; hd < H + G; hd += NT / 64) {
+    float* x = qk + hd * D;
+    for (int f = lane; f < half; f += 64) {
+      const int i0 = pairs ? 2 * f : f, i1 = pairs ? 2 * f + 1 : f + half;
+      const float a = x[i0], b = x[i1], c = cs[f], sn = cs[half + f];
+      x[i0] = a * c - b * sn;
+      x[i1] = b * c + a * sn;
+    }
+  }
+  __syncthreads();
   if (slot >= 0) {
     AT* kd = kc + slot * Ck;
-    for (int g = wave; g < G; g += NT / 64)
-      for (int dh = lane; dh < D; dh += 64) stf(kd + g * D + dh, elem(row + Cq + g * D, dh));
-    AT* vd = vt + (slot / PAGE) * (int64_t)Cv * PAGE + (slot % PAGE);
-    for (int i = threadIdx.x; i < Cv; i += NT) stf(vd + (int64_t)i * PAGE, ldf(row + Cq + Ck + i));
+    for (int i = threadIdx.x; i < Ck; i += NT) stf(kd + i, qk[Cq + i]);
   }
-  if (talk == nullptr) return;
-  float* tsh = qsh + Cq;
-  for (int i = threadIdx.x; i < H * H; i += NT) tsh[i] = talk[i];
-  __syncthreads();
-  // a wave per (head h, key head c): its rep mix weights are wave-uniform, lanes run over the key head's dimensions
+  if (talk == nullptr) {
+    for (int i = threadIdx.x; i < Cq; i += NT) stf(q_out + t * qos + i, qk[i]);
+    return;
+  }
   const int rep = H / G;
+  if (rep <= MIX_REP) {
+    // a wave per (key head c, 64 of its dimensions): the rep query values of a lane's dimension stay in registers for
+    // all H outputs; the weights are wave-uniform (broadcast) LDS reads, rep per output, all requested before the
+    // multiply-adds
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    const int nb = (D + 63) >> 6;
+    for (int task = wv; task < G * nb; task += NT / 64) {
+      const int c = task / nb, i = ((task - c * nb) << 6) + lane;
+      // (loads at clamped, always valid addresses and a select afterwards: nothing between them that would make the
+      // compiler wait for one LDS read before it issues the next)
+      const int ic = min(i, D - 1);
+      float qv[MIX_REP];
+#pragma unroll
+      for (int r = 0; r < MIX_REP; ++r) {
+        const float v = qk[(c * rep + min(r, rep - 1)) * D + ic];
+        qv[r] = (r < rep && i < D) ? v : 0.f;
+      }
+      for (int h = 0; h < H; ++h) {
+        const float* tr = tsh + h * H + c * rep;
+        float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+        for (int r0 = 0; r0 < MIX_REP; r0 += 8) {
+          if (r0 < rep) {   // (uniform) eight weights requested together; query values past rep are zero
+            float wt[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) wt[j] = tr[min(r0 + j, rep - 1)];
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+              v0 += wt[j] * qv[r0 + j];
+              v1 += wt[j + 1] * qv[r0 + j + 1];
+            }
+          }
+        }
+        if (i < D) stf(q_out + t * qos + ((int64_t)h * G + c) * D + i, v0 + v1);
+      }
+    }
+    return;
+  }
   for (int hc = wave; hc < H * G; hc += NT / 64) {
     const int h = hc / G, c = hc - h * G;
     const float* tr = tsh + h * H + c * rep;
     for (int i = lane; i < D; i += 64) {
-      const float* qp = qsh + (c * rep) * D + i;
-      float v0 = 0.f, v1 = 0.f;
-      for (int r0 = 0; r0 < rep; r0 += 8) {   // eight weights and eight query values requested before the first use
-        float tv[8], qv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int r = min(r0 + j, rep - 1);
-          tv[j] = r0 + j < rep ? tr[r] : 0.f;
-          qv[j] = qp[r * D];
-        }
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          v0 += tv[j] * qv[j];
-          v1 += tv[j + 1] * qv[j + 1];
-        }
-      }
-      stf(q_out + t * qos + (int64_t)hc * D + i, v0 + v1);
+      const float* qp = qk + (c * rep) * D + i;
+      float v = 0.f;
+      for (int r = 0; r < rep; ++r) v += tr[r] * qp[r * D];
+      stf(q_out + t * qos + (int64_t)hc * D + i, v);
     }
   }
 }
@@ -534,7 +572,7 @@ hipError_t kafka_hy_hgrn2_combine(const int* cs, int R, const float* F, int HD, 
   return hipGetLastError();
 }
 
-int kafka_hy_rope_store_max_q() { return 11264; }   // H D floats of LDS when the queries are mixed (+ H H <= 4096)
+int kafka_hy_rope_store_max_q() { return 15360; }   // floats of LDS: H D + G D + rot dims (+ H H with a head mix)
 
 hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, int G, int D, int Dv,
                                   const int64_t* positions, const float* cos_sin, int dims, int pairs,
@@ -542,8 +580,9 @@ hipError_t kafka_hy_rope_kv_store(int f32, const void* qkv, int64_t qs, int H, i
                                   int64_t T, hipStream_t st) {
   if (T <= 0) return hipSuccess;
   if (dims < 0 || dims % 2 || dims > D || (dims > 0 && cos_sin == nullptr) || G < 1 || H % G) return hipErrorInvalidValue;
-  if (talk != nullptr && (H * D > kafka_hy_rope_store_max_q() || H > 64)) return hipErrorInvalidValue;
-  const size_t lds = talk != nullptr ? (size_t)(H * D + H * H) * sizeof(float) : 0;
+  const int64_t fl = (int64_t)(H + G) * D + dims + (talk != nullptr ? H * H : 0);
+  if (fl > kafka_hy_rope_store_max_q()) return hipErrorInvalidValue;
+  const size_t lds = (size_t)fl * sizeof(float);
   DISPATCH_AT(f32, {
     rope_kv_store_kernel<AT><<<(unsigned)T, NT, lds, st>>>((const AT*)qkv, qs, H, G, D, Dv, positions, cos_sin, dims,
                                                            pairs != 0, talk, (AT*)kc, (AT*)vt, slots, (AT*)q_out, qos);

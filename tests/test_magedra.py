@@ -204,6 +204,26 @@ def test_row_ops(device):
     assert close(both[:, 40:], want, 1e-5)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,off", [(64, 16), (4096, 8), (40, 13), (72, 0)])
+def test_row_ops_bf16_vectors(n, off):
+    """The bf16 forms of the gate and of the clamped activation: sizes and offsets that take 8-element vectors and
+    ones that do not, outputs into column slices."""
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(n)
+    T = 9
+    a = torch.randn(T, n, generator=g).to(torch.bfloat16)
+    gate = torch.randn(T, off + n + 8, generator=g).to(torch.bfloat16)
+    both = torch.zeros(T, n + 16, dtype=torch.bfloat16, device=dev)
+    hops.gate_mul(a.to(dev), gate.to(dev), off, 0.7, both[:, :n])
+    want = a.double() * torch.sigmoid(gate[:, off:off + n].double()) * 0.7
+    assert close(both[:, :n].float(), want, 1e-2) and float(both[:, n:].abs().max()) == 0.0
+    gu = (2.0 * torch.randn(T, 2 * n, generator=g)).to(torch.bfloat16)
+    hops.swish_clamp_mul(gu.to(dev), 1.3, 1.702, both[:, 8:8 + n])
+    gg, uu = gu[:, :n].double().clamp(max=1.3), gu[:, n:].double().clamp(-1.3, 1.3)
+    assert close(both[:, 8:8 + n].float(), gg * torch.sigmoid(1.702 * gg) * (uu + 1.0), 1e-2)
+
+
 PORTIONS = [[(0, 9), (1, 2)], [(1, 1), (0, 1)], [(0, 2), (1, 3)], [(1, 7)], [(0, 130), (1, 65)], [(0, 1)], [(1, 201), (0, 3)]]
 
 

@@ -368,8 +368,8 @@ __global__ void hgrn2_combine_kernel(const int* __restrict__ cs, const float* __
 
 // ---- attention inputs: rotation, head mix, paged store -------------------------------------------------------------------
 // One workgroup per row of the fused projection [q (H D) | k (G D) | v (G Dv) | ...]. The row's q and k parts, the
-// position's cos | sin row and the mix matrix are staged in LDS as fp32 in one round of independent loads (a step of few
-// rows is one memory round trip per row); pairs are rotated in place (a thread owns both members); keys leave for
+// position's cos | sin row and the mix matrix are staged in LDS as fp32 in one batch of independent loads (a step of few
+// rows pays one memory latency per row); pairs are rotated in place (a thread owns both members); keys leave for
 // their page; the queries leave as they are, or with `talk` as q'[h][c D + i] = sum_r talk[h][c rep + r] q[c rep + r][i]
 // (rep = H / G).
 constexpr int MIX_REP = 32;   // query heads per key head whose values a lane keeps in registers for the head mix
